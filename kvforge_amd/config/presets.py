@@ -149,6 +149,70 @@ PRESETS["rudorax-1b"] = rudorax_stack(vocab=128256, width=2048, pairs=8, heads=3
                                       experts=32, top=4, identity=2, shared_ff=2048)
 
 
+def buzinex(vocab: int, width: int, layers: list, embedding_scale: float = 1.0, logit_scale: float = 1.0,
+            logit_softcap: float | None = None, eps: float = 1e-6,
+            max_positions: int | None = None) -> dict[str, Any]:
+    """A Buzinex config.json.  ``layers``: one ``(type, mixer, ff)`` per layer.  For
+    ``"attention"`` the mixer holds ``heads kv_heads dim vdim scale`` and optionally ``softcap``,
+    ``q_temp`` (``(coef, every)``) and ``window``; for ``"latent_attention"`` ``heads dim
+    rot_dim vdim kv_rank scale`` and optionally ``window`` and ``base``; for ``"wkv"`` ``heads
+    dim decay_rank``.  ``ff``: the feed-forward's width, or ``None`` for none."""
+    out = []
+    for kind, m, ff in layers:
+        if kind == "attention":
+            qt = m.get("q_temp")
+            mixer: dict[str, Any] = {
+                "dim": m["dim"], "heads": m["heads"], "kv_heads": m["kv_heads"],
+                "q_temp": {"coef": float(qt[0]), "every": int(qt[1])} if qt else None,
+                "scale": float(m["scale"]), "softcap": m.get("softcap"), "vdim": m["vdim"]}
+            if m.get("window"):
+                mixer["mask"] = {"size": m["window"]}
+        elif kind == "latent_attention":
+            mixer = {"dim": m["dim"], "heads": m["heads"], "kv_rank": m["kv_rank"],
+                     "mask": {"size": m["window"]} if m.get("window") else None,
+                     "rot": ({"base": float(m.get("base", 10000.0)), "dims": m.get("rot_dims", m["rot_dim"])}
+                             if m["rot_dim"] else None),
+                     "rot_dim": m["rot_dim"], "scale": float(m["scale"]), "vdim": m["vdim"]}
+        else:
+            mixer = {"decay_rank": m["decay_rank"], "dim": m["dim"], "heads": m["heads"]}
+        out.append({"mixer": mixer, "mlp": {"ff": ff, "kind": "dense"} if ff else None, "type": kind})
+    cfg: dict[str, Any] = {
+        "architecture": "Buzinex", "embedding": {"scale": float(embedding_scale)}, "layers": out,
+        "logit_scale": float(logit_scale), "logit_softcap": logit_softcap, "norm": {"eps": eps},
+        "vocab": vocab, "width": width}
+    if max_positions is not None:
+        cfg["max_positions"] = max_positions
+    return cfg
+
+
+def buzinex_stack(vocab: int, width: int, groups: int, heads: int, kv_heads: int, dim: int, latent_dim: int,
+                  rot_dim: int, kv_rank: int, window: int, wkv_heads: int, wkv_dim: int, ff: int,
+                  max_positions: int = 131072) -> dict[str, Any]:
+    """``groups`` times (capped attention, latent attention, wkv without a feed-forward, latent
+    attention), the attention layers with dense feed-forwards."""
+    att = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=float(dim) ** -0.5, softcap=50.0,
+               q_temp=(0.1, 4096))
+    lat = dict(heads=heads, dim=latent_dim, rot_dim=rot_dim, vdim=latent_dim, kv_rank=kv_rank,
+               scale=float(latent_dim + rot_dim) ** -0.5, window=window, base=1000000.0)
+    rec = dict(heads=wkv_heads, dim=wkv_dim, decay_rank=64)
+    return buzinex(vocab, width, [("attention", att, ff), ("latent_attention", lat, ff), ("wkv", rec, None),
+                                  ("latent_attention", lat, ff)] * groups,
+                   embedding_scale=float(width) ** 0.5, logit_scale=float(width) ** -0.5, logit_softcap=30.0,
+                   max_positions=max_positions)
+
+
+PRESETS["buzinex-tiny"] = buzinex(
+    vocab=320, width=96,
+    layers=[("attention", dict(heads=4, kv_heads=2, dim=16, vdim=32, scale=0.25, softcap=20.0, q_temp=(0.3, 8)), 160),
+            ("latent_attention", dict(heads=3, dim=16, rot_dim=8, vdim=24, kv_rank=40, scale=0.2, window=24), 160),
+            ("wkv", dict(heads=2, dim=24, decay_rank=8), None)],
+    embedding_scale=8.0, logit_scale=0.5, logit_softcap=20.0, max_positions=1024)
+# layers of the width of llama-1b: what this design's kernels are measured at
+PRESETS["buzinex-1b"] = buzinex_stack(vocab=128256, width=2048, groups=4, heads=32, kv_heads=8, dim=64,
+                                      latent_dim=64, rot_dim=32, kv_rank=192, window=1024, wkv_heads=32,
+                                      wkv_dim=64, ff=8192)
+
+
 def preset_dict(name: str) -> dict[str, Any]:
     try:
         return dict(PRESETS[name])

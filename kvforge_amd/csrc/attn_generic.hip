@@ -30,7 +30,11 @@ struct AttnArgs {
   float scale;
   const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
   const float* sinks;   // null, or one number per q head: exp(sinks[h]) joins the softmax's denominator (a key without a value)
+  float cap;            // 0, or the scaled score s becomes cap * tanh(s / cap)
 };
+
+// the scaled score under the cap (0: none)
+__device__ __forceinline__ float capped(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -177,7 +181,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
           const int j = t0 + 16 * st + 4 * g4 + v;
           bool vis = row_ok && j <= pos && j < ctx;
           if (a.window > 0) vis = vis && (j > pos - a.window || j < keep);
-          sc[v] = vis ? fmaf(slope, static_cast<float>(j - pos), sc[v] * a.scale) : -INFINITY;
+          sc[v] = vis ? fmaf(slope, static_cast<float>(j - pos), capped(sc[v] * a.scale, a.cap)) : -INFINITY;
           tmax = fmaxf(tmax, sc[v]);
         }
         p[st] = sc;
@@ -302,6 +306,7 @@ struct DecodeArgs {
   float scale;
   const float* slopes;  // as in AttnArgs
   const float* sinks;   // as in AttnArgs
+  float cap;            // as in AttnArgs
 };
 
 // GT: heads of the group handled together (a power of two, at most 8; a larger group is taken
@@ -401,7 +406,7 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
     float corr[GT];
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
-      const float sc = (vis && page >= 0) ? fmaf(slope[g], static_cast<float>(j - pos), s[g] * a.scale) : -INFINITY;
+      const float sc = (vis && page >= 0) ? fmaf(slope[g], static_cast<float>(j - pos), capped(s[g] * a.scale, a.cap)) : -INFINITY;
       const float m_new = fmaxf(m_run[g], wave_max(sc));
       float p = 0.f;
       corr[g] = 1.f;
@@ -582,13 +587,14 @@ KVF_EXPORT int kvf_attn_generic_decode(int dtype, const void* q, const void* k_p
                                        int H, int KV, int d, int block_size, int num_blocks,
                                        int table_stride, int q_stride, int o_stride, int window,
                                        int keep, int n_seqs, int splits, float scale,
-                                       const float* slopes, const float* sinks, hipStream_t s) {
+                                       const float* slopes, const float* sinks, float cap, hipStream_t s) {
   if (num_seqs <= 0) return 0;
+  if (!(cap >= 0.f)) return static_cast<int>(hipErrorInvalidValue);
   if (keep < 0 || d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || splits < 1 ||
       (splits > 1 && (!part_acc || !part_ml)) || block_size <= 0)
     return static_cast<int>(hipErrorInvalidValue);
   DecodeArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-               splits, keep, scale, slopes, sinks};
+               splits, keep, scale, slopes, sinks, cap};
   if (dtype == 0)
     return launch_decode<float>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,
                                 part_acc, part_ml, num_seqs, a, s);
@@ -606,12 +612,13 @@ KVF_EXPORT int kvf_attn_generic(int dtype, const void* q, const void* k_pages, c
                                 const int* work, int num_work, void* out, int H, int KV, int d,
                                 int block_size, int num_blocks, int table_stride, int q_stride,
                                 int o_stride, int window, int keep, int n_seqs, float scale,
-                                const float* slopes, const float* sinks, hipStream_t s) {
+                                const float* slopes, const float* sinks, float cap, hipStream_t s) {
+  if (!(cap >= 0.f)) return static_cast<int>(hipErrorInvalidValue);
   if (keep < 0 || d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || !work || block_size <= 0 ||
       q_stride % 4 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
   AttnArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-             keep, scale, slopes, sinks};
+             keep, scale, slopes, sinks, cap};
   if (dtype == 0)
     return launch<float>(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, out, a, s);
   if (dtype == 1)

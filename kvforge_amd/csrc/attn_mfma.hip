@@ -81,6 +81,7 @@ struct MArgs {
   // null, or one number per q head: exp(sinks[h]) joins the softmax's denominator, a key without
   // a value whose score is not scaled
   const float* sinks;
+  float cap;  // 0, or the scaled score s becomes cap * tanh(s / cap) (kernels with BIAS == 2)
 };
 
 // A walk over the blocks of 32 keys that a range of rows sees: blocks counted from `first` up to
@@ -205,15 +206,16 @@ template <int RT> struct Rows {
 
 // One key block for the row tiles of a wave: scores, lazy softmax update, P * V.
 // References live in log2 units: scale2 = scale * log2(e) > 0 is applied inside the exponent.
-// BIAS: a score also gets its head's slope times the key's distance from the row's position;
-// the scores are then brought to log2 units before the maximum is taken.
-template <int DT, int RT, bool BIAS>
+// BIAS 1: a score also gets its head's slope times the key's distance from the row's position;
+// the scores are then brought to log2 units before the maximum is taken.  BIAS 2: the scaled
+// score s becomes cap * tanh(s / cap), likewise before the maximum.
+template <int DT, int RT, int BIAS>
 __device__ __forceinline__ void block_update(const bf16x8 (&kf)[2][(DT + 1) / 2], const bf16x8 (&vf)[DT],
                                              const bf16x8 (&qf)[RT][(DT + 1) / 2], const Rows<RT>& rows,
                                              int kb, int kg, bool edge, float scale_log2, float (&m_ref)[RT], float (&l_run)[RT],
-                                             f32x4 (&acc)[RT][DT]) {
+                                             f32x4 (&acc)[RT][DT], float cap = 0.f) {
   constexpr int DC = (DT + 1) / 2;
-  const float scale2 = BIAS ? 1.f : scale_log2;
+  const float scale2 = BIAS != 0 ? 1.f : scale_log2;
   f32x4 s[RT][2];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
@@ -224,6 +226,15 @@ __device__ __forceinline__ void block_update(const bf16x8 (&kf)[2][(DT + 1) / 2]
       for (int c = 0; c < DC; ++c)
         s[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][c], qf[rt][c], s[rt][t], 0, 0, 0);
     }
+  if constexpr (BIAS == 2) {
+    const float in = scale_log2 / (LOG2E * cap), out = cap * LOG2E;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[rt][t][r] = out * tanhf(s[rt][t][r] * in);
+  }
   // lane holds keys kb + 8*kg + 4*t + r of its row
   if (edge) {
 #pragma unroll
@@ -237,7 +248,7 @@ __device__ __forceinline__ void block_update(const bf16x8 (&kf)[2][(DT + 1) / 2]
           s[rt][t][r] = vis ? s[rt][t][r] : -INFINITY;
         }
   }
-  if constexpr (BIAS) {
+  if constexpr (BIAS == 1) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const float at0 = rows.slope2[rt] * static_cast<float>(kb + 8 * kg - rows.pos[rt]);
@@ -346,7 +357,7 @@ __device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int 
 // SHARE: the waves stage the fragments of each key block in LDS for each other; otherwise every
 // wave loads all of them itself.
 // SINK: the softmax has a sink (a.sinks); a kernel without is the code it was before sinks came
-template <int DT, int RT, bool SHARE, bool BIAS, bool SINK>
+template <int DT, int RT, bool SHARE, int BIAS, bool SINK>
 __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
@@ -492,7 +503,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 #pragma unroll
         for (int t = 0; t < DT; ++t) vf[t] = as_frag(frag_lds[(buf * N_FRAG + N_K + t) * KVF_WAVE + lane]);
         const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
-        block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+        block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
       }
     };
     const int kb_first = wk.first;
@@ -576,7 +587,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 #pragma unroll
       for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(vr[t], vl));
       const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
-      block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+      block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
     }
   }
 
@@ -602,7 +613,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 // ------------------------------------------------------------------------- few rows, split keys
 // TWO: a wave holds the fragments of two blocks, loading one while it consumes the other.
 // NW: waves of the workgroup; more of them shorten each wave's walk over its cut of the keys.
-template <int DT, bool TWO, int NW, bool BIAS, bool SINK>
+template <int DT, bool TWO, int NW, int BIAS, bool SINK>
 __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
@@ -690,7 +701,7 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
 #pragma unroll
     for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(r.v[t], r.vl));
     const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
-    block_update<DT, 1, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+    block_update<DT, 1, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
   };
   // Without a window the page lookups of the first blocks are asked for together with the
   // query and the context length, not after them: one round trip to memory less.
@@ -859,18 +870,23 @@ void launch_runs_rt(dim3 grid, hipStream_t s, const void* q, const void* k_pages
   constexpr bool SHARE = runs_share(DT);
   constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
   const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
-  if (a.sinks)   // (never with slopes: the exported entry refuses the pair)
-    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, false, true>), grid, dim3(256), lds, s,
+  if (a.cap > 0.f)   // (never with sinks or slopes: the exported entry refuses the pairs)
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, 2, false>), grid, dim3(256), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), a);
+  else if (a.sinks)   // (never with slopes: the exported entry refuses the pair)
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, 0, true>), grid, dim3(256), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), a);
   else if (a.slopes)
-    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, true, false>), grid, dim3(256), lds, s,
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, 1, false>), grid, dim3(256), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), a);
   else
-    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, false, false>), grid, dim3(256), lds, s,
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, 0, false>), grid, dim3(256), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), a);
@@ -894,18 +910,23 @@ void launch_split_waves(dim3 grid, hipStream_t s, const void* q, const void* k_p
                         const int* block_table, const int* seq_ids, const int* cu_q, const int* ctx_lens,
                         void* out, float* part_acc, float* part_ml, const MArgs& a) {
   const size_t lds = (static_cast<size_t>(NW) * DT * KVF_WAVE * 4 + NW * 16 * 2) * sizeof(float);
-  if (a.sinks)
-    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, false, true>), grid, dim3(NW * KVF_WAVE), lds, s,
+  if (a.cap > 0.f)
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, 2, false>), grid, dim3(NW * KVF_WAVE), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), part_acc, part_ml, a);
+  else if (a.sinks)
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, 0, true>), grid, dim3(NW * KVF_WAVE), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), part_acc, part_ml, a);
   else if (a.slopes)
-    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, true, false>), grid, dim3(NW * KVF_WAVE), lds, s,
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, 1, false>), grid, dim3(NW * KVF_WAVE), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), part_acc, part_ml, a);
   else
-    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, false, false>), grid, dim3(NW * KVF_WAVE), lds, s,
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, 0, false>), grid, dim3(NW * KVF_WAVE), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), part_acc, part_ml, a);
@@ -951,7 +972,7 @@ int runs_blocks_per_cu() {
   constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
   const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
   int n = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attn_mfma_runs_kernel<DT, RT, SHARE, false, false>, 256, lds) !=
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attn_mfma_runs_kernel<DT, RT, SHARE, 0, false>, 256, lds) !=
       hipSuccess)
     return 0;
   return n;
@@ -980,9 +1001,11 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
                                      const int* work, int num_work, int rows_per_item, void* out, int H, int KV, int d,
                                      int bs, int nb, int table_stride, int q_stride, int o_stride,
                                      int window, int keep, int n_seqs, float scale, const float* slopes,
-                                     const void* gate, int gate_stride, const float* sinks, hipStream_t s) {
+                                     const void* gate, int gate_stride, const float* sinks, float cap,
+                                     hipStream_t s) {
   if (num_work <= 0) return 0;
   if (sinks && slopes) return static_cast<int>(hipErrorInvalidValue);   // no kernel has both
+  if (!(cap >= 0.f) || (cap > 0.f && (sinks || slopes))) return static_cast<int>(hipErrorInvalidValue);
   if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
     return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0)
@@ -994,7 +1017,7 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
   // of one head and finds them in its own L2 after the first workgroup has brought them in.
   const int kv_fastest = num_work <= 65535 ? 1 : 0;
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, keep, kv_fastest, scale, magic_of(bs), slopes,
-                static_cast<const bf16_t*>(gate), gate_stride, sinks};
+                static_cast<const bf16_t*>(gate), gate_stride, sinks, cap};
   const dim3 grid = kv_fastest ? dim3(KV, num_work) : dim3(num_work, KV);
   switch (d / 16) {
 #define GO(DT) \
@@ -1014,16 +1037,18 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
                                     int num_seqs, int H, int KV, int d, int bs, int nb,
                                     int table_stride, int q_stride, int o_stride, int window,
                                     int keep, int n_seqs, int splits, float scale, const float* slopes,
-                                    const void* gate, int gate_stride, const float* sinks, hipStream_t s) {
+                                    const void* gate, int gate_stride, const float* sinks, float cap,
+                                    hipStream_t s) {
   if (num_seqs <= 0) return 0;
   if (sinks && slopes) return static_cast<int>(hipErrorInvalidValue);
+  if (!(cap >= 0.f) || (cap > 0.f && (sinks || slopes))) return static_cast<int>(hipErrorInvalidValue);
   if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
     return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||
       splits > KVF_WAVE || (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, keep, 0, scale, magic_of(bs), slopes,
-                static_cast<const bf16_t*>(gate), gate_stride, sinks};
+                static_cast<const bf16_t*>(gate), gate_stride, sinks, cap};
   const int G = H / KV, chunks = (G + 15) / 16;
   if (num_seqs > 65535) return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid(KV * chunks, num_seqs, splits);

@@ -535,12 +535,17 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_kernel(
     T* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ block_table, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    const float* __restrict__ qw, const float* __restrict__ kw, int dk, float eps, RopeArgs a) {
+    const float* __restrict__ qw, const float* __restrict__ kw, int dk, float eps, float qt_coef,
+    int qt_every, RopeArgs a) {
   const int n = blockIdx.x;
   const int p = positions[n];
   const int half = a.rot / 2;
   T* row = qkv + static_cast<size_t>(n) * a.row_len;
   const bool pos_ok = p >= 0 && p < a.table_len;
+  // query temperature: q heads are stretched by 1 + coef * ln(floor((p + 1) / every) + 1)
+  const float q_temp = qt_every > 0 && p >= 0
+                           ? 1.f + qt_coef * logf(static_cast<float>((p + 1) / qt_every) + 1.f)
+                           : 1.f;
   const float* cs = cos_t ? cos_t + static_cast<size_t>(pos_ok ? p : 0) * half : nullptr;
   const float* sn = sin_t ? sin_t + static_cast<size_t>(pos_ok ? p : 0) * half : nullptr;
   int page = -1, off = 0;
@@ -569,7 +574,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_kernel(
       v[j] = e + 1 < dk ? Elem<T>::load(x + e + 1) : 0.f;
       ss = fmaf(u[j], u[j], fmaf(v[j], v[j], ss));
     }
-    const float r = 1.f / sqrtf(wave_sum(ss) / static_cast<float>(dk) + eps);
+    const float r = (is_k ? 1.f : q_temp) / sqrtf(wave_sum(ss) / static_cast<float>(dk) + eps);
     T* dst = is_k ? k_pages + ((static_cast<size_t>(page) * a.KV + (hh - a.H)) * a.block_size + off) * a.d : x;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -598,8 +603,8 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_kernel(
 template <typename T>
 static int qknorm_rope_launch(void* qkv, const int* positions, const int* seq_of_token, const float* cos_t,
                               const float* sin_t, const int* block_table, void* k_pages, void* v_pages,
-                              const float* qw, const float* kw, int dk, float eps, int n, RopeArgs a,
-                              hipStream_t s) {
+                              const float* qw, const float* kw, int dk, float eps, float qt_coef,
+                              int qt_every, int n, RopeArgs a, hipStream_t s) {
   if (n <= 0) return 0;
   if (a.d > 4 * KVF_WAVE || dk > a.d || dk <= 0 || a.rot > dk || a.rot % 2 || !qw || (a.write_kv && !kw))
     return static_cast<int>(hipErrorInvalidValue);
@@ -609,35 +614,38 @@ static int qknorm_rope_launch(void* qkv, const int* positions, const int* seq_of
   if (shares > 64) shares = 64;
   hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, dim3(n, shares), dim3(256), 0, s, static_cast<T*>(qkv), positions,
                      seq_of_token, cos_t, sin_t, block_table, static_cast<T*>(k_pages),
-                     static_cast<T*>(v_pages), qw, kw, dk, eps, a);
+                     static_cast<T*>(v_pages), qw, kw, dk, eps, qt_coef, qt_every, a);
   return kvf_last_error();
 }
 #define QKNORM_ARGS_DECL                                                                         \
   void *qkv, const int *positions, const int *seq_of_token, const float *cos_t,                 \
       const float *sin_t, const int *block_table, void *k_pages, void *v_pages, const float *qw, \
-      const float *kw, int dk, float eps, int n, int H, int KV, int d, int rot, int table_len,   \
+      const float *kw, int dk, float eps, float qt_coef, int qt_every, int n, int H, int KV,    \
+      int d, int rot, int table_len,                                                             \
       int block_size, int table_stride, int num_blocks, int write_kv, int n_seqs, int row_len,   \
       hipStream_t s
 KVF_EXPORT int kvf_qknorm_rope_kvwrite_f32(QKNORM_ARGS_DECL) {
   return qknorm_rope_launch<float>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
-                                   v_pages, qw, kw, dk, eps, n, ROPE_ARGS_PACK, s);
+                                   v_pages, qw, kw, dk, eps, qt_coef, qt_every, n, ROPE_ARGS_PACK, s);
 }
 KVF_EXPORT int kvf_qknorm_rope_kvwrite_bf16(QKNORM_ARGS_DECL) {
   return qknorm_rope_launch<bf16_t>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
-                                    v_pages, qw, kw, dk, eps, n, ROPE_ARGS_PACK, s);
+                                    v_pages, qw, kw, dk, eps, qt_coef, qt_every, n, ROPE_ARGS_PACK, s);
 }
 
 // ----------------------------------------------------------------------------- soft cap
-// x = cap * tanh(x / cap) over fp32 values (logits), in place.
-__global__ void softcap_kernel(float* __restrict__ x, long total, float cap) {
+// x = cap * tanh(x * scale / cap) over fp32 values (logits), in place; cap 0: x = x * scale.
+__global__ void softcap_kernel(float* __restrict__ x, long total, float cap, float scale) {
   const long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < total) x[i] = cap * tanhf(x[i] / cap);
+  if (i >= total) return;
+  const float v = x[i] * scale;
+  x[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
 }
-KVF_EXPORT int kvf_softcap(float* x, long total, float cap, hipStream_t s) {
+KVF_EXPORT int kvf_softcap(float* x, long total, float cap, float scale, hipStream_t s) {
   if (total <= 0) return 0;
-  if (!(cap > 0.f)) return static_cast<int>(hipErrorInvalidValue);
+  if (!(cap >= 0.f)) return static_cast<int>(hipErrorInvalidValue);
   hipLaunchKernelGGL(softcap_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, s, x,
-                     total, cap);
+                     total, cap, scale);
   return kvf_last_error();
 }
 

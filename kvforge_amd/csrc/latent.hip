@@ -1,0 +1,155 @@
+// Latent attention: what lies between the projections and the paged attention kernels.
+//
+// A token's keys and values of all heads are read out of one latent vector c [rank] (RMS-normed)
+// and one rotated key part k_r [rot] that the heads share.  With W_uk the read-out of the
+// unrotated keys, q_h . (W_uk_h c) = (W_uk_h^T q_h) . c, so attention runs over ONE key per
+// token, [k_r | c], with per-head queries [q_r_h | W_uk_h^T q_h]; the weighted sum of the c is
+// taken by the same kernels (the value is the key's c part) and read out per head by W_uv_h
+// afterwards.  The cache holds k_r and c and nothing per head.
+//
+//   latent_split : a projected row [q heads (dim | rot) ... | c_raw (rank) | k_r (rot)] becomes
+//                  the attention kernels' row [H q heads | k | v] of heads of d elements:
+//                  q head h = [q_r_h | (left for head_product) | 0], k = [k_r | norm(c) | 0],
+//                  v = [0 | norm(c) | 0]; the norm in fp32 with one rounding.
+//   head_product : out[n, h, :] = W[h] in[n, h, :] for per-head matrices W [H, O, I]
+//                  (fp32 multiply and add on the vector ALUs, tiles of 32 rows x 64 outputs
+//                  through LDS).
+#include "common.h"
+
+namespace {
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_split_kernel(const T* __restrict__ proj, int ld_in,
+                                                           T* __restrict__ qkv, int ld_out,
+                                                           const float* __restrict__ w, float eps, int H,
+                                                           int dim, int rot, int rank, int d) {
+  __shared__ float scratch[16];
+  const int n = blockIdx.x, tid = threadIdx.x;
+  const T* in = proj + static_cast<size_t>(n) * ld_in;
+  T* out = qkv + static_cast<size_t>(n) * ld_out;
+  const T* down = in + H * (dim + rot);
+  float ss = 0.f;
+  for (int i = tid; i < rank; i += blockDim.x) {
+    const float v = Elem<T>::load(down + i);
+    ss = fmaf(v, v, ss);
+  }
+  const float r = 1.f / sqrtf(block_sum(ss, scratch) / static_cast<float>(rank) + eps);
+  // q heads: the rotated part to the front, zeros behind what head_product fills
+  for (int i = tid; i < H * d; i += blockDim.x) {
+    const int h = i / d, e = i - h * d;
+    if (e < rot)
+      out[i] = in[h * (dim + rot) + dim + e];
+    else if (e >= rot + rank || dim == 0)   // (heads without a plain part: nothing fills the middle)
+      Elem<T>::store(out + i, 0.f);
+  }
+  T* k = out + H * d;
+  T* v = k + d;
+  for (int e = tid; e < d; e += blockDim.x) {
+    if (e < rot) {
+      k[e] = down[rank + e];
+      Elem<T>::store(v + e, 0.f);
+    } else if (e < rot + rank) {
+      const float c = Elem<T>::load(down + e - rot) * r * w[e - rot];
+      Elem<T>::store(k + e, c);
+      Elem<T>::store(v + e, c);
+    } else {
+      Elem<T>::store(k + e, 0.f);
+      Elem<T>::store(v + e, 0.f);
+    }
+  }
+}
+
+constexpr int HP_M = 32, HP_N = 64, HP_K = 32;
+
+// grid (row tiles, output tiles, heads); 256 threads, thread (ty, tx) owns rows ty, ty + 16 and
+// outputs tx + 16 j (j = 0..3) of the tile.
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void head_product_kernel(const T* __restrict__ in, int ld_in, int in_head,
+                                                           const TW* __restrict__ W, T* __restrict__ out,
+                                                           int ld_out, int out_head, int N, int O, int I) {
+  __shared__ float As[HP_M][HP_K + 1];
+  __shared__ float Bs[HP_N][HP_K + 1];
+  const int n0 = blockIdx.x * HP_M, o0 = blockIdx.y * HP_N, h = blockIdx.z;
+  const int tid = threadIdx.x, ty = tid / 16, tx = tid % 16;
+  const T* a = in + static_cast<size_t>(h) * in_head;
+  const TW* w = W + static_cast<size_t>(h) * O * I;
+  float acc[2][4] = {};
+  for (int k0 = 0; k0 < I; k0 += HP_K) {
+    for (int i = tid; i < HP_M * HP_K; i += 256) {
+      const int r = i / HP_K, c = i % HP_K;
+      As[r][c] = (n0 + r < N && k0 + c < I) ? Elem<T>::load(a + static_cast<size_t>(n0 + r) * ld_in + k0 + c) : 0.f;
+    }
+    for (int i = tid; i < HP_N * HP_K; i += 256) {
+      const int r = i / HP_K, c = i % HP_K;
+      Bs[r][c] = (o0 + r < O && k0 + c < I) ? Elem<TW>::load(w + static_cast<size_t>(o0 + r) * I + k0 + c) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < HP_K; ++c) {
+      const float a0 = As[ty][c], a1 = As[ty + 16][c];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float b = Bs[tx + 16 * j][c];
+        acc[0][j] = fmaf(a0, b, acc[0][j]);
+        acc[1][j] = fmaf(a1, b, acc[1][j]);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int n = n0 + ty + 16 * i;
+    if (n >= N) continue;
+    T* o = out + static_cast<size_t>(n) * ld_out + static_cast<size_t>(h) * out_head;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (o0 + tx + 16 * j < O) Elem<T>::store(o + o0 + tx + 16 * j, acc[i][j]);
+  }
+}
+
+template <typename T, typename TW>
+int head_product_launch(const void* in, int ld_in, int in_head, const void* W, void* out, int ld_out,
+                        int out_head, int N, int H, int O, int I, hipStream_t s) {
+  const dim3 grid((N + HP_M - 1) / HP_M, (O + HP_N - 1) / HP_N, H);
+  hipLaunchKernelGGL((head_product_kernel<T, TW>), grid, dim3(256), 0, s, static_cast<const T*>(in), ld_in, in_head,
+                     static_cast<const TW*>(W), static_cast<T*>(out), ld_out, out_head, N, O, I);
+  return kvf_last_error();
+}
+}  // namespace
+
+// dtype: 0 = fp32, 1 = bf16 (rows in and out).  d >= rot + rank.
+KVF_EXPORT int kvf_latent_split(int dtype, const void* proj, int ld_in, void* qkv, int ld_out, const float* w,
+                                float eps, int n, int H, int dim, int rot, int rank, int d, hipStream_t s) {
+  if (n <= 0) return 0;
+  if (H <= 0 || dim < 0 || rot < 0 || rank <= 0 || d < rot + rank || ld_in < H * (dim + rot) + rank + rot ||
+      ld_out < (H + 2) * d || !w)
+    return static_cast<int>(hipErrorInvalidValue);
+  if (dtype == 0)
+    hipLaunchKernelGGL(latent_split_kernel<float>, dim3(n), dim3(256), 0, s, static_cast<const float*>(proj), ld_in,
+                       static_cast<float*>(qkv), ld_out, w, eps, H, dim, rot, rank, d);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(latent_split_kernel<bf16_t>, dim3(n), dim3(256), 0, s, static_cast<const bf16_t*>(proj), ld_in,
+                       static_cast<bf16_t*>(qkv), ld_out, w, eps, H, dim, rot, rank, d);
+  else
+    return static_cast<int>(hipErrorInvalidValue);
+  return kvf_last_error();
+}
+
+// out[n, h * out_head + o] = sum_i W[h, o, i] * in[n * ld_in + h * in_head + i]; dtype of rows
+// and wtype of W: 0 = fp32, 1 = bf16.
+KVF_EXPORT int kvf_head_product(int dtype, int wtype, const void* in, int ld_in, int in_head, const void* W,
+                                void* out, int ld_out, int out_head, int N, int H, int O, int I,
+                                hipStream_t s) {
+  if (N <= 0) return 0;
+  if (H <= 0 || O <= 0 || I <= 0 || H > 65535 || (O + HP_N - 1) / HP_N > 65535)
+    return static_cast<int>(hipErrorInvalidValue);
+  if (dtype == 0 && wtype == 0)
+    return head_product_launch<float, float>(in, ld_in, in_head, W, out, ld_out, out_head, N, H, O, I, s);
+  if (dtype == 1 && wtype == 1)
+    return head_product_launch<bf16_t, bf16_t>(in, ld_in, in_head, W, out, ld_out, out_head, N, H, O, I, s);
+  if (dtype == 1 && wtype == 0)
+    return head_product_launch<bf16_t, float>(in, ld_in, in_head, W, out, ld_out, out_head, N, H, O, I, s);
+  if (dtype == 0 && wtype == 1)
+    return head_product_launch<float, bf16_t>(in, ld_in, in_head, W, out, ld_out, out_head, N, H, O, I, s);
+  return static_cast<int>(hipErrorInvalidValue);
+}

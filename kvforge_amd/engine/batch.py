@@ -197,6 +197,10 @@ class Step:
         # library product over many rows leaves it here instead of running an add kernel; the
         # next norm adds it on its way (``take_owed``), anything else calls ``settle`` first.
         self.owed: tuple[torch.Tensor, torch.Tensor] | None = None
+        # Rows that a block has handed to a sublayer in place of the stream and that hold
+        # nothing yet: the sublayer's last product is written there instead of added
+        # (``parts.base.add_product``), which then forgets the mark.
+        self.fresh: torch.Tensor | None = None
         # the staging memory this step was filled from (``fill_step``), for ``upload_ints``
         self._meta: "MetaBuffers | None" = None
         self._turn = 0

@@ -46,6 +46,8 @@ MODULES: dict[str, list[str]] = {
     "gemm_library": ["gemm_library.hip"],
     "mlstm": ["mlstm.hip"],
     "moe": ["moe.hip"],
+    "latent": ["latent.hip"],
+    "wkv": ["wkv.hip"],
 }
 
 

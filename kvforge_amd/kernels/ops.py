@@ -112,13 +112,14 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: floa
     _ok(f(ids.data_ptr(), table.data_ptr(), out.data_ptr(), n, h, vocab, float(scale), _stream()), "embed")
 
 
-def softcap(x: torch.Tensor, cap: float) -> None:
-    """``x = cap * tanh(x / cap)`` in place over fp32 values (logits)."""
+def softcap(x: torch.Tensor, cap: float | None, scale: float = 1.0) -> None:
+    """``x = cap * tanh(x * scale / cap)`` in place over fp32 values (logits); without a cap
+    (``None``) ``x = x * scale``."""
     _check(x, "x", F32)
-    if not cap > 0.0:
+    if cap is not None and not cap > 0.0:
         raise KernelError(f"softcap: the cap must be positive, got {cap}")
-    f = _fn("elementwise", "kvf_softcap", [c_void_p, c_long, c_float, c_void_p])
-    _ok(f(x.data_ptr(), x.numel(), float(cap), _stream()), "softcap")
+    f = _fn("elementwise", "kvf_softcap", [c_void_p, c_long, c_float, c_float, c_void_p])
+    _ok(f(x.data_ptr(), x.numel(), float(cap or 0.0), float(scale), _stream()), "softcap")
 
 
 # ------------------------------------------------------------------------------ RMS norm
@@ -439,11 +440,14 @@ def qknorm_rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token
                         cos: torch.Tensor | None, sin: torch.Tensor | None, block_table: torch.Tensor,
                         k_pages: torch.Tensor, v_pages: torch.Tensor, num_heads: int,
                         num_kv_heads: int, head_dim: int, q_weight: torch.Tensor,
-                        k_weight: torch.Tensor, norm_dim: int, eps: float, write_kv: bool = True) -> None:
+                        k_weight: torch.Tensor, norm_dim: int, eps: float, write_kv: bool = True,
+                        q_temp: tuple[float, int] | None = None) -> None:
     """``rope_kvwrite`` with a norm per head in front of the rotation: every q and k head is
     divided by the root mean square of its first ``norm_dim`` elements (``eps`` inside the root)
     and multiplied by ``q_weight`` / ``k_weight`` (fp32 ``[norm_dim]``, shared by the heads), in
-    fp32 from the projected row; elements ``norm_dim..head_dim-1`` (padding) stay zero."""
+    fp32 from the projected row; elements ``norm_dim..head_dim-1`` (padding) stay zero.
+    ``q_temp = (coef, every)``: the q heads of a token at position ``p`` are also multiplied by
+    ``1 + coef * ln(floor((p + 1) / every) + 1)``."""
     n = qkv.shape[0]
     H, KV, d = num_heads, num_kv_heads, head_dim
     _check(qkv, "qkv", None, (n, None))
@@ -466,10 +470,13 @@ def qknorm_rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token
     nb, _, bs, _ = k_pages.shape
     _check(v_pages, "v_pages", qkv.dtype, (nb, KV, d, bs))
     f = _fn("elementwise", f"kvf_qknorm_rope_kvwrite_{_suffix(qkv.dtype)}",
-            [c_void_p] * 10 + [c_int, c_float] + [c_int] * 12 + [c_void_p])
+            [c_void_p] * 10 + [c_int, c_float, c_float, c_int] + [c_int] * 12 + [c_void_p])
+    coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
+    if q_temp is not None and every < 1:
+        raise KernelError(f"qknorm_rope_kvwrite: q_temp's step must be positive, got {every}")
     _ok(f(qkv.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), cos_p, sin_p,
           block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), q_weight.data_ptr(),
-          k_weight.data_ptr(), int(norm_dim), float(eps), n, H, KV, d, rot, table_len, bs, stride, nb,
+          k_weight.data_ptr(), int(norm_dim), float(eps), coef, every, n, H, KV, d, rot, table_len, bs, stride, nb,
           1 if write_kv else 0, n_seqs, qkv.shape[1], _stream()), "qknorm_rope_kvwrite")
 
 
@@ -964,6 +971,17 @@ def _no_sinks_with_slopes(sinks, slopes, on_matrix_cores: bool) -> None:
         raise KernelError("attention: the matrix-core kernels take sinks or slopes, not both")
 
 
+def _score_cap(cap, sinks, slopes, on_matrix_cores: bool) -> float:
+    """The cap on scaled scores as the kernels take it (0: none)."""
+    if cap is None:
+        return 0.0
+    if not cap > 0.0:
+        raise KernelError(f"attention: the score cap must be positive, got {cap}")
+    if on_matrix_cores and (sinks is not None or slopes is not None):
+        raise KernelError("attention: the matrix-core kernels cap scores without sinks and slopes only")
+    return float(cap)
+
+
 def _keep_first(window: int, keep_first: int) -> int:
     """Keys kept visible behind a window; without a window every key is visible anyway."""
     keep = int(keep_first)
@@ -1019,7 +1037,7 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  head_dim: int, scale: float, window: int = 0,
                  slopes: torch.Tensor | None = None, rows_per_item: int | None = None,
                  keep_first: int = 0, gate: torch.Tensor | None = None,
-                 sinks: torch.Tensor | None = None) -> None:
+                 sinks: torch.Tensor | None = None, score_cap: float | None = None) -> None:
     """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 3]`` rows
     (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
     an item covers ``rows_per_item`` of them (what ``prefill_rows_per_item`` gave when the rows
@@ -1032,9 +1050,12 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     attention output times ``sigmoid(gate)``, element by element, in the matrix-core kernels'
     store (the 32-bit kernels take no gate: their caller runs ``sigmoid_gate`` behind them).
     ``sinks``: fp32 ``[H]``; the softmax's denominator of head ``h`` then holds one more term
-    ``exp(sinks[h])``, a key without a value whose score is not scaled."""
+    ``exp(sinks[h])``, a key without a value whose score is not scaled.
+    ``score_cap``: the scaled score ``s`` becomes ``score_cap * tanh(s / score_cap)`` (the
+    matrix-core kernels have it without sinks and slopes only)."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
+    cap = _score_cap(score_cap, sinks, slopes, attention_on_matrix_cores(q.dtype, k_pages.shape[2]))
     _check(work, "work", I32, (None, 3))
     keep = _keep_first(window, keep_first)
     gp, gs = _gate_args(gate, q, H * d)
@@ -1046,11 +1067,11 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     _no_sinks_with_slopes(sinks, slopes, attention_on_matrix_cores(q.dtype, bs))
     if attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
-                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p])
+                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p])
         _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
               cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(), work.shape[0], int(rows_per_item), out.data_ptr(),
               H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window), keep,
-              n_seqs, float(scale), sl, gp, gs, sk, _stream()), "attn_mfma_prefill")
+              n_seqs, float(scale), sl, gp, gs, sk, cap, _stream()), "attn_mfma_prefill")
         return
     if gate is not None:
         raise KernelError("attn_prefill: the 32-bit kernel takes no gate; gate its rows afterwards")
@@ -1061,11 +1082,11 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         raise KernelError("attn_prefill: rows of q and out must start on 16 bytes")
     f = _fn("attn_generic", "kvf_attn_generic",
             [c_int] + [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 11
-            + [c_float, c_void_p, c_void_p, c_void_p])
+            + [c_float, c_void_p, c_void_p, c_float, c_void_p])
     _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
           block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(),
           work.shape[0], out.data_ptr(), H, KV, d, bs, nb, block_table.shape[1], q.stride(0),
-          out.stride(0), int(window), keep, n_seqs, float(scale), sl, sk, _stream()), "attn_generic")
+          out.stride(0), int(window), keep, n_seqs, float(scale), sl, sk, cap, _stream()), "attn_generic")
 
 
 def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -1075,7 +1096,7 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
                 token_is_seq: bool = False, slopes: torch.Tensor | None = None,
                 keep_first: int = 0, gate: torch.Tensor | None = None,
-                sinks: torch.Tensor | None = None) -> None:
+                sinks: torch.Tensor | None = None, score_cap: float | None = None) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
     each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  The key
     range may be cut into ``splits`` runs; ``workspace`` then holds fp32 partial accumulators
@@ -1084,9 +1105,10 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     single tokens), which spares the matrix-core kernel a dependent load.  ``slopes``: as in
     ``attn_prefill``; ``keep_first`` and ``gate`` likewise (the matrix-core kernels only: the
     32-bit path is given no gate, its caller gates the rows afterwards); ``sinks`` likewise (all
-    kernels; with cuts the term joins the sum where the cuts are merged)."""
+    kernels; with cuts the term joins the sum where the cuts are merged); ``score_cap`` likewise."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
+    cap = _score_cap(score_cap, sinks, slopes, attention_on_matrix_cores(q.dtype, k_pages.shape[2]))
     sl = _slopes_ptr(slopes, H, q)
     sk = _sinks_ptr(sinks, H, q)
     keep = _keep_first(window, keep_first)
@@ -1116,23 +1138,23 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         if gate is not None:
             raise KernelError("attn_decode: the 32-bit kernel takes no gate; gate its rows afterwards")
         f = _fn("attn_generic", "kvf_attn_generic_decode",
-                [c_int] + [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p, c_void_p])
+                [c_int] + [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p, c_float, c_void_p])
         _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
               block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
               None if token_is_seq else cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
               pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
               num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
-              int(window), keep, n_seqs, int(splits), float(scale), sl, sk, _stream()), "attn_generic_decode")
+              int(window), keep, n_seqs, int(splits), float(scale), sl, sk, cap, _stream()), "attn_generic_decode")
         return
     f = _fn("attn_mfma", "kvf_attn_mfma_decode",
-            [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p])
+            [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p])
     _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
           seq_ids.data_ptr() if seq_ids is not None else None,
           None if token_is_seq else cu_q.data_ptr(),
           ctx_lens.data_ptr(), out.data_ptr(), pa.data_ptr() if pa is not None else None,
           pm.data_ptr() if pm is not None else None, num_seqs, H, KV, d, bs, nb,
           block_table.shape[1], q.stride(0), out.stride(0), int(window), keep, n_seqs, int(splits),
-          float(scale), sl, gp, gs, sk, _stream()), "attn_mfma_decode")
+          float(scale), sl, gp, gs, sk, cap, _stream()), "attn_mfma_decode")
 
 
 # ------------------------------------------------------------------------------ matrix-memory recurrence
@@ -1263,6 +1285,145 @@ def mlstm_out(heads_raw: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor,
     f = _fn("mlstm", "kvf_mlstm_out", [c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p] + [c_int] * 3 + [c_void_p])
     _ok(f(_tcode(out.dtype), heads_raw.data_ptr(), gate.data_ptr(), gate.stride(0) if n > 1 else H * dv,
           weight.data_ptr(), float(eps), out.data_ptr(), n, H, dv, _stream()), "mlstm_out")
+
+
+# ------------------------------------------------------------------------------ latent attention
+def latent_split(proj: torch.Tensor, qkv: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                 heads: int, dim: int, rot: int, rank: int, head_dim: int) -> None:
+    """A projected row ``[heads x (dim | rot) | latent (rank) | shared key part (rot)]`` becomes
+    the attention kernels' row ``[heads + 2, head_dim]``: q head ``h`` gets its ``rot`` part in
+    front (columns ``rot..rot+rank-1`` are left for ``head_product`` to fill, the rest is
+    zero), the one k head is ``[key part | norm(latent) | 0]`` and the one v head
+    ``[0 | norm(latent) | 0]``, the norm being ``x / sqrt(mean(x^2) + eps) * norm_weight`` in
+    fp32 with one rounding."""
+    n = proj.shape[0]
+    H, d = int(heads), int(head_dim)
+    _check(proj, "proj", None, (n, None), contiguous=False)
+    _check(qkv, "qkv", proj.dtype, (n, (H + 2) * d))
+    _check(norm_weight, "norm_weight", F32, (rank,))
+    if proj.stride(1) != 1 or proj.shape[1] < H * (dim + rot) + rank + rot or d < rot + rank:
+        raise KernelError(f"latent_split: rows of {proj.shape[1]} elements / heads of {d} do not hold "
+                          f"{H} x ({dim} + {rot}) + {rank} + {rot}")
+    f = _fn("latent", "kvf_latent_split", [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_float]
+            + [c_int] * 6 + [c_void_p])
+    _ok(f(_tcode(proj.dtype), proj.data_ptr(), proj.stride(0) if n > 1 else proj.shape[1], qkv.data_ptr(),
+          qkv.shape[1], norm_weight.data_ptr(), float(eps), n, H, int(dim), int(rot), int(rank), d,
+          _stream()), "latent_split")
+
+
+def head_product(x: torch.Tensor, in_head: int, w: torch.Tensor, out: torch.Tensor, out_head: int) -> None:
+    """``out[n, h * out_head + o] = sum_i w[h, o, i] * x[n, h * in_head + i]`` for per-head
+    matrices ``w [H, O, I]``: ``x`` and ``out`` are rows (views of wider rows are fine) in which
+    head ``h`` starts ``h * in_head`` / ``h * out_head`` elements in.  fp32 multiply and add."""
+    n = x.shape[0]
+    _check(w, "w", None, (None, None, None))
+    H, O, I = w.shape
+    _check(x, "x", None, (n, None), contiguous=False)
+    _check(out, "out", x.dtype, (n, None), contiguous=False)
+    if x.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("head_product: rows must be dense")
+    if (H - 1) * in_head + I > x.shape[1] or (H - 1) * out_head + O > out.shape[1] or in_head < 0 or out_head < 0:
+        raise KernelError(f"head_product: {H} heads of {I} / {O} elements do not fit rows of "
+                          f"{x.shape[1]} / {out.shape[1]}")
+    if _overlap(x, out):
+        raise KernelError("head_product: out must not share memory with x")
+    f = _fn("latent", "kvf_head_product", [c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p]
+            + [c_int] * 6 + [c_void_p])
+    _ok(f(_tcode(x.dtype), _tcode(w.dtype), x.data_ptr(), x.stride(0) if n > 1 else x.shape[1], int(in_head),
+          w.data_ptr(), out.data_ptr(), out.stride(0) if n > 1 else out.shape[1], int(out_head), n, H, O, I,
+          _stream()), "head_product")
+
+
+# ------------------------------------------------------------------------------ decaying matrix memory
+def wkv_state_floats(heads: int, dim: int, width: int) -> int:
+    """fp32 numbers of a request's slot: every head's ``S [dim, dim]``, then the last input row."""
+    return heads * dim * dim + width
+
+
+def wkv_mix(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, prev_off: int, slot_ids: torch.Tensor,
+            seq_of_token: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor, out: torch.Tensor,
+            n_seqs: int) -> None:
+    """``out[m, t] = h[t] + (h_prev[t] - h[t]) * mu[m]`` for ``mu [M, width]`` (fp32): ``h_prev``
+    is the row before ``t`` in its query run, for a run's first token the row kept at
+    ``prev_off`` in the sequence's state slot (zeros at position 0 or without a slot); the last
+    row of every run is left in its slot."""
+    n, width = h.shape
+    _check(h, "h", None, (n, width))
+    _check(mu, "mu", F32, (None, width))
+    M = mu.shape[0]
+    _check(out, "out", h.dtype, (M, n, width))
+    _check(state, "state", F32, (None, None))
+    for t, name in ((slot_ids, "slot_ids"), (seq_of_token, "seq_of_token"), (cu_q, "cu_q"), (positions, "positions")):
+        _check(t, name, I32, (None,))
+    if seq_of_token.shape[0] < n or positions.shape[0] < n or cu_q.shape[0] < n_seqs + 1 or slot_ids.shape[0] < n_seqs:
+        raise KernelError("wkv_mix: batch arrays shorter than the batch")
+    if prev_off < 0 or prev_off + width > state.shape[1]:
+        raise KernelError("wkv_mix: the kept row does not fit the slot")
+    f = _fn("wkv", "kvf_wkv_mix", [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int] + [c_void_p] * 5
+            + [c_int] * 5 + [c_void_p])
+    _ok(f(_tcode(h.dtype), h.data_ptr(), mu.data_ptr(), state.data_ptr(), state.shape[1], int(prev_off),
+          slot_ids.data_ptr(), seq_of_token.data_ptr(), cu_q.data_ptr(), positions.data_ptr(), out.data_ptr(),
+          width, M, int(n_seqs), state.shape[0], n, _stream()), "wkv_mix")
+
+
+def tanh_cast(x: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = tanh(x)`` for fp32 ``x``, rounded once to ``out``'s type."""
+    _check(x, "x", F32)
+    _check(out, "out", None, tuple(x.shape))
+    f = _fn("wkv", "kvf_wkv_tanh", [c_int, c_void_p, c_void_p, c_long, c_void_p])
+    _ok(f(_tcode(out.dtype), x.data_ptr(), out.data_ptr(), x.numel(), _stream()), "tanh_cast")
+
+
+def wkv_scan(rows: torch.Tensor, r_off: int, k_off: int, v_off: int, z: torch.Tensor, w0: torch.Tensor,
+             u: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Tensor,
+             state: torch.Tensor, out: torch.Tensor, n_seqs: int, heads: int, dim: int) -> None:
+    """The recurrence ``o_j = sum_i r_i (S_ij + u_i k_i v_j)``, ``S_ij <- w_i S_ij + k_i v_j`` with
+    ``w = exp(-exp(z + w0))`` over every query run, token by token in fp32, from and to the
+    sequences' state slots (a run at position 0 starts from zeros whatever its slot holds; a
+    sequence without a slot starts from zeros and keeps nothing).  ``rows``: r, k, v of a
+    token ``[heads * dim]`` each at the given offsets of its row; ``z`` fp32 ``[n, >= heads *
+    dim]``; ``w0``, ``u`` fp32 ``[heads * dim]``; ``out`` fp32 ``[n, heads * dim]``."""
+    n = rows.shape[0]
+    H, dk = int(heads), int(dim)
+    _check(rows, "rows", None, (n, None))
+    if max(r_off, k_off, v_off) + H * dk > rows.shape[1] or min(r_off, k_off, v_off) < 0:
+        raise KernelError("wkv_scan: r, k, v do not fit the rows")
+    _check(z, "z", F32, (n, None))
+    if z.shape[1] < H * dk:
+        raise KernelError("wkv_scan: decay rows too short")
+    _check(w0, "w0", F32, (H * dk,))
+    _check(u, "u", F32, (H * dk,))
+    _check(out, "out", F32, (n, H * dk))
+    _check(state, "state", F32, (None, None))
+    if state.shape[1] < H * dk * dk or not 0 < dk <= 256:
+        raise KernelError(f"wkv_scan: heads of {dk} (at most 256) need slots of {H * dk * dk} floats")
+    for t, name in ((cu_q, "cu_q"), (positions, "positions"), (slot_ids, "slot_ids")):
+        _check(t, name, I32, (None,))
+    if cu_q.shape[0] < n_seqs + 1 or slot_ids.shape[0] < n_seqs or positions.shape[0] < n:
+        raise KernelError("wkv_scan: batch arrays shorter than the batch")
+    f = _fn("wkv", "kvf_wkv_scan", [c_int] + [c_void_p] * 9 + [c_int] * 10 + [c_void_p])
+    _ok(f(_tcode(rows.dtype), rows.data_ptr(), z.data_ptr(), w0.data_ptr(), u.data_ptr(), cu_q.data_ptr(),
+          positions.data_ptr(), slot_ids.data_ptr(), state.data_ptr(), out.data_ptr(), int(n_seqs), H, dk,
+          state.shape[0], state.shape[1], rows.shape[1], int(r_off), int(k_off), int(v_off), z.shape[1],
+          _stream()), "wkv_scan")
+
+
+def wkv_out(heads_raw: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float,
+            out: torch.Tensor, heads: int, dim: int) -> None:
+    """``out[n, h, :] = o / rms(o) * weight[h, :] * silu(gate[n, h, :])`` for the raw heads
+    ``o = heads_raw[n, h, :]`` (fp32), the root mean square per head with ``eps`` inside the
+    root.  ``gate``: dense rows of ``out``'s type (a view of wider rows is fine)."""
+    n = heads_raw.shape[0]
+    H, dk = int(heads), int(dim)
+    _check(heads_raw, "heads_raw", F32, (n, H * dk))
+    _check(weight, "weight", F32, (H * dk,))
+    _check(out, "out", None, (n, H * dk))
+    _check(gate, "gate", out.dtype, (n, H * dk), contiguous=False)
+    if gate.stride(1) != 1:
+        raise KernelError("wkv_out: gate rows must be dense")
+    f = _fn("wkv", "kvf_wkv_out", [c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p] + [c_int] * 3 + [c_void_p])
+    _ok(f(_tcode(out.dtype), heads_raw.data_ptr(), gate.data_ptr(), gate.stride(0) if n > 1 else H * dk,
+          weight.data_ptr(), float(eps), out.data_ptr(), n, H, dk, _stream()), "wkv_out")
 
 
 # ------------------------------------------------------------------------------ routed experts

@@ -97,7 +97,12 @@ class PagedAttention(Mixer):
     kernel that also rotates and writes the cache.
     ``sink``: name of a tensor ``[num_heads]`` under the prefix: the softmax's denominator of
     head ``h`` gets one more term ``exp(sink[h])`` (not scaled), which takes weight from the
-    keys and has no value."""
+    keys and has no value.
+    ``score_cap``: the scaled score ``s`` becomes ``score_cap * tanh(s / score_cap)`` before
+    mask and softmax.
+    ``q_temp``: ``(coef, every)``; the query of position ``p`` is multiplied by
+    ``1 + coef * ln(floor((p + 1) / every) + 1)``, in the kernel that norms q and k (so it goes
+    with ``qk_norm``)."""
 
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "g": "g_proj.weight"}
@@ -110,7 +115,8 @@ class PagedAttention(Mixer):
                  window: int | None = None, score_slopes=None, keep_first: int = 0,
                  value_dim: int | None = None, gated: bool = False, own_kv: bool = True,
                  names: dict[str, str] | None = None,
-                 qk_norm: tuple[str, str, float] | None = None, sink: str | None = None) -> None:
+                 qk_norm: tuple[str, str, float] | None = None, sink: str | None = None,
+                 score_cap: float | None = None, q_temp: tuple[float, int] | None = None) -> None:
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.dk = int(head_dim)
@@ -140,6 +146,12 @@ class PagedAttention(Mixer):
         if qk_norm is not None and not own_kv:
             raise ValueError("a norm of q and k goes with key and value projections of the mixer's own")
         self.q_norm_w = self.k_norm_w = self.sinks = None
+        self.score_cap = float(score_cap) if score_cap else None
+        if self.score_cap is not None and not self.score_cap > 0.0:
+            raise ValueError(f"score_cap must be positive, got {score_cap}")
+        self.q_temp = (float(q_temp[0]), int(q_temp[1])) if q_temp else None
+        if self.q_temp is not None and (qk_norm is None or self.q_temp[1] < 1):
+            raise ValueError("q_temp goes with qk_norm and a positive step")
         self.cache_spec = CacheSpec(attention_pages(self.KV, self.d), self.window, self.keep_first)
         self.w_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
@@ -359,7 +371,7 @@ class PagedAttention(Mixer):
                 ops.qknorm_rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
                                         layer.k_pages, layer.v_pages, H, KV, d, self.q_norm_w,
                                         self.k_norm_w, self.dk, self.qk_norm[2],
-                                        write_kv=layer.owns_cache)
+                                        write_kv=layer.owns_cache, q_temp=self.q_temp)
             elif self.own_kv or self.rotary is not None:
                 ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
                                  layer.k_pages, layer.v_pages, H, KV, d,
@@ -374,7 +386,8 @@ class PagedAttention(Mixer):
         if work is not None:
             ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
                              work, out, H, KV, d, self.scale, window, self.slopes, rows_per_item,
-                             keep_first=self.keep_first, gate=gate_in_kernel, sinks=self.sinks)
+                             keep_first=self.keep_first, gate=gate_in_kernel, sinks=self.sinks,
+                             score_cap=self.score_cap)
         if step.n_decode:
             splits = self._decode_cuts(step, ops.attention_on_matrix_cores(act, bs))
             workspace = None
@@ -386,7 +399,7 @@ class PagedAttention(Mixer):
                             window, splits, workspace,
                             token_is_seq=step.decode_seq_ids is None and work is None,
                             slopes=self.slopes, keep_first=self.keep_first, gate=gate_in_kernel,
-                            sinks=self.sinks)
+                            sinks=self.sinks, score_cap=self.score_cap)
         if gate is not None and gate_in_kernel is None:
             ops.sigmoid_gate(out, gate)
         add_product(step, out, self.w_o, residual, owed=owed)

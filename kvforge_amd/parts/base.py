@@ -23,9 +23,11 @@ class WeightSpec:
     """One checkpoint tensor a part expects.
 
     ``init`` drives the random-weights mode: ``"normal"`` draws N(0, std), ``"norm"`` draws
-    1 + N(0, std), ``"zeros"`` is zero.  ``integer`` tensors are tables of int32."""
+    1 + N(0, std), ``"zeros"`` is zero.  ``integer`` tensors are tables of int32.  A size of
+    ``None`` is one that the checkpoint decides (the part reads it off the tensor it is handed);
+    random weights cannot be drawn for such a spec."""
 
-    shape: tuple[int, ...]
+    shape: tuple
     init: str = "normal"
     std: float = 0.02
     integer: bool = False
@@ -174,6 +176,11 @@ class Norm(Part):
         ``rows`` the sum is left in ``x``."""
         raise NotImplementedError
 
+    def add_to(self, stream: torch.Tensor, y: torch.Tensor) -> None:
+        """``stream += norm(y)`` for fp32 rows ``y`` of the stream's shape (a norm behind a
+        sublayer, whose output joins the stream only after it)."""
+        raise NotImplementedError
+
 
 class Positions(Part):
     """Position encoding.  Two hooks, both optional: one on the embedding output (absolute
@@ -307,9 +314,18 @@ def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.
     is cut into two halves of K so that every compute unit pulls on the weight: the first half
     is added here, the second is left owed (rounded to bf16, as a stored product is).
     ``owed``: a sum the caller took from the step (``step.take_owed``) and has not added yet;
-    it is added here, in the same kernel where that is possible."""
+    it is added here, in the same kernel where that is possible.
+    A ``residual`` that the step holds as *fresh* (``step.fresh``: a sublayer's own output rows,
+    which a block norms before they join the stream) is written, not added to: the product is
+    stored there in fp32 whatever kernel makes it, and nothing is left owed."""
     from kvforge_amd.kernels import ops
 
+    if getattr(step, "fresh", None) is residual:
+        step.fresh = None
+        ops.gemm(a, w, residual)
+        if owed is not None:
+            ops.add_rows(residual, owed)
+        return
     if ops.is_library_product(a, w):
         if owed is not None:
             ops.add_rows(residual, owed)

@@ -148,3 +148,48 @@ class ParallelBlock(Block):
                 bias = self.ffn.down_bias
         if self.after is not None:
             self.after.forward(residual, step, bias=bias)
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """A norm before and after each sublayer: ``x += post(mixer(pre(x)))`` and then, if the layer
+    has a feed-forward, ``x += ffn_post(ffn(ffn_pre(x)))``.  A sublayer's output does not join
+    the stream as it is, so its last product is written to rows of its own (fp32; the step
+    holds them as ``fresh``, see ``parts.base.add_product``), and the norm behind the sublayer
+    adds them to the stream (``Norm.add_to``: norm and sum in one pass, in fp32)."""
+
+    def __init__(self, pre: Norm, mixer: Mixer, post: Norm, ffn_pre: Norm | None = None,
+                 ffn: FeedForward | None = None, ffn_post: Norm | None = None) -> None:
+        if ffn is not None and (ffn_pre is None or ffn_post is None):
+            raise ValueError("a feed-forward in a sandwich block needs its two norms")
+        self.pre, self.mixer, self.post = pre, mixer, post
+        self.ffn_pre, self.ffn, self.ffn_post = (ffn_pre, ffn, ffn_post) if ffn is not None else (None, None, None)
+
+    def parts(self) -> list[Part]:
+        return [p for p in (self.pre, self.mixer, self.post, self.ffn_pre, self.ffn, self.ffn_post)
+                if p is not None]
+
+    def kernel_modules(self, dtype) -> set[str]:
+        return super().kernel_modules(dtype) | {"elementwise"}
+
+    def forward(self, residual, step, layer: LayerState) -> None:
+        shape = tuple(residual.shape)
+        x = step.ws.buf("normed", shape, step.act_dtype)
+        self.pre.forward(residual, x, add=step.take_owed(residual))
+        branch = step.ws.buf("sublayer_out", shape, torch.float32)
+        step.fresh = branch
+        self.mixer.forward(x, step, layer, branch)
+        self._join(residual, branch, self.post, step)
+        if self.ffn is None:
+            return
+        self.ffn_pre.forward(residual, x)
+        step.fresh = branch
+        self.ffn.forward(x, step, branch)
+        self._join(residual, branch, self.ffn_post, step)
+
+    @staticmethod
+    def _join(residual, branch, post: Norm, step) -> None:
+        if step.fresh is branch:
+            raise RuntimeError("a sublayer of a sandwich block must end in parts.base.add_product")
+        step.settle()
+        post.add_to(residual, branch)

@@ -45,15 +45,19 @@ class TokenEmbedding(Embedding):
 class LMHead(Head):
     """``logits = x @ W^T`` in fp32 output.  ``tied_to``: the checkpoint name of the embedding
     table when the head shares it (then no tensor of its own is expected).  ``tensor``: the
-    matrix's whole checkpoint name where it is not ``<prefix>.weight``.  ``softcap``: the logits
-    become ``softcap * tanh(logits / softcap)`` (``None``: as they are)."""
+    matrix's whole checkpoint name where it is not ``<prefix>.weight``.  ``scale``: the logits are
+    multiplied by it.  ``softcap``: the (scaled) logits become ``softcap * tanh(logits /
+    softcap)`` (``None``: as they are)."""
 
     replayable = True
 
     def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: str | None = None,
-                 tensor: str | None = None, softcap: float | None = None) -> None:
+                 tensor: str | None = None, softcap: float | None = None, scale: float = 1.0) -> None:
         self.prefix, self.vocab, self.hidden, self.tied_to = prefix, int(vocab), int(hidden), tied_to
         self.softcap = float(softcap) if softcap else None
+        self.scale = float(scale)
+        if not self.scale > 0.0:
+            raise ValueError(f"the logits' scale must be positive, got {scale}")
         self.tensor = tied_to if tied_to is not None else (tensor if tensor is not None else self._name("weight"))
         self.weight: torch.Tensor | None = None
 
@@ -65,7 +69,7 @@ class LMHead(Head):
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         return ({"gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
-                | ({"elementwise"} if self.softcap else set()))
+                | ({"elementwise"} if self.softcap or self.scale != 1.0 else set()))
 
     def num_bytes(self) -> int:
         w = ops.plain_of(self.weight)
@@ -80,8 +84,8 @@ class LMHead(Head):
 
     def forward(self, x: torch.Tensor, logits: torch.Tensor) -> None:
         ops.gemm(x, self.weight, logits)
-        if self.softcap:
-            ops.softcap(logits, self.softcap)
+        if self.softcap or self.scale != 1.0:
+            ops.softcap(logits, self.softcap, self.scale)
 
     def can_pick(self, rows: int) -> bool:
         """Whether ``pick`` takes so many rows with this weight.  Never under a soft cap: where

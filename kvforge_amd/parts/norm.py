@@ -38,6 +38,11 @@ class RMSNorm(Norm):
                 add: torch.Tensor | None = None) -> None:
         ops.rmsnorm(x, self.weight, self.eps, out, rows, add)
 
+    def add_to(self, stream: torch.Tensor, y: torch.Tensor) -> None:
+        if self.weight.dtype != torch.float32:
+            self.weight = self.weight.float()    # the kernel multiplies by an fp32 vector
+        ops.rms_add(stream, y, self.weight, self.eps)
+
     def foldable_into(self, matrix: torch.Tensor) -> bool:
         """Whether this norm's weight may be multiplied into the columns of a bf16 matrix: only
         when it is itself held in bf16 (a weight stored in 32-bit stays a 32-bit multiply)."""
@@ -60,6 +65,26 @@ class OnePlusRMSNorm(RMSNorm):
 
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
         self.weight = (1.0 + tensors[self.name].float()).contiguous()
+
+    def foldable_into(self, matrix: torch.Tensor) -> bool:
+        return False
+
+
+@register_norm("rmsnorm_named")
+class NamedRMSNorm(RMSNorm):
+    """RMS norm with a plain weight vector that the checkpoint holds under ``name`` (the whole
+    name, no ``.weight`` behind it).  The weight is kept in fp32, so the product with it is a
+    32-bit one in every mode."""
+
+    def __init__(self, name: str, width: int, eps: float) -> None:
+        super().__init__("", width, eps)
+        self.name = name
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self.name: WeightSpec((self.width,), init="norm", std=0.1)}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.name].float().contiguous()
 
     def foldable_into(self, matrix: torch.Tensor) -> bool:
         return False

@@ -30,7 +30,8 @@ def check_index(expected: dict[str, WeightSpec], index: dict[str, tuple], ignore
         if name not in index:
             continue
         _, shape, dt = index[name]
-        if tuple(shape) != tuple(spec.shape):
+        if len(shape) != len(spec.shape) or any(want is not None and want != got
+                                                  for want, got in zip(spec.shape, shape)):
             wrong.append(f"{name}: expected {list(spec.shape)}, found {list(shape)}")
         elif spec.integer and dt not in _INT_STORED:
             wrong.append(f"{name}: expected an integer table, found {dt}")

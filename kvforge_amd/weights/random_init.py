@@ -27,6 +27,12 @@ def _stored_as(dtype: "str | torch.dtype") -> torch.dtype:
         raise ValueError(f"random weights are stored as bfloat16 or float32, not {dtype!r}") from None
 
 
+def _sized(name: str, w) -> None:
+    if any(s is None for s in w.shape):
+        raise ValueError(f"{name}: a size that only a checkpoint decides ({list(w.shape)}); a random "
+                         f"model's configuration has to give it")
+
+
 def random_tensors(spec, seed: int, dtype: "str | torch.dtype" = "bfloat16") -> dict[str, torch.Tensor]:
     """Tensors for every name the model expects, drawn in 32-bit in sorted name order from one
     generator and stored as ``dtype`` (the reference draws in 32-bit and casts to the engine's
@@ -35,6 +41,7 @@ def random_tensors(spec, seed: int, dtype: "str | torch.dtype" = "bfloat16") -> 
     gen = torch.Generator().manual_seed(int(seed))
     out: dict[str, torch.Tensor] = {}
     for name, w in sorted(spec.weight_specs().items()):
+        _sized(name, w)
         if w.integer:
             out[name] = torch.zeros(w.shape, dtype=torch.int32)
         elif w.init == "zeros":
@@ -75,6 +82,7 @@ def load_random_weights(spec, seed: int, engine_dtype: torch.dtype, device: "tor
     gen = torch.Generator(device=device).manual_seed(int(seed))
     tensors: dict[str, torch.Tensor] = {}
     for name, w in sorted(spec.weight_specs().items()):
+        _sized(name, w)
         if w.integer:
             tensors[name] = torch.zeros(w.shape, dtype=torch.int32, device=device)
             continue

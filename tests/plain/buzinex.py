@@ -59,6 +59,23 @@ def softmax_rows(scores: torch.Tensor, visible: torch.Tensor, sink: torch.Tensor
     return e / den
 
 
+def visible_keys(queries: int, keys: int, window: int | None = None) -> torch.Tensor:
+    """``[queries, keys]``: the queries are the last ``queries`` of ``keys`` positions; position
+    ``i`` sees ``j <= i`` and, under a window, only ``i - j < window``."""
+    i = torch.arange(keys - queries, keys)[:, None]
+    j = torch.arange(keys)[None, :]
+    seen = j <= i
+    return seen & (i - j < int(window)) if window else seen
+
+
+def attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, visible: torch.Tensor,
+           cap: float | None = None, sink: torch.Tensor | None = None) -> torch.Tensor:
+    """``q [Tq, H, d]``, ``k [Tk, H, d]``, ``v [Tk, H, dv]`` -> ``[Tq, H, dv]``: scores scaled,
+    capped, masked, softmax (with a sink, if any), weighted sum."""
+    s = capped(torch.einsum("thd,shd->hts", q, k) * float(scale), cap)
+    return torch.einsum("hts,shd->thd", softmax_rows(s, visible, sink), v)
+
+
 # ---------------------------------------------------------------------------------- attention
 def query_temperature(positions: torch.Tensor, coef: float, every: int) -> torch.Tensor:
     """``1 + coef * ln(floor((p + 1) / every) + 1)`` per position, in 32-bit."""
@@ -88,12 +105,9 @@ def attention(h: torch.Tensor, w: dict, p: str, m: dict, eps: float,
     q, k = stored(q, store), stored(k, store)
     k = k.repeat_interleave(H // G, dim=1)
     v = v.repeat_interleave(H // G, dim=1)
-    s = torch.einsum("thd,shd->hts", q, k) * float(m["scale"])
-    s = capped(s, m.get("softcap"))
-    visible = pos[None, :] <= pos[:, None]
-    a = softmax_rows(s, visible)
-    o = stored(torch.einsum("hts,shd->thd", a, v).reshape(T, H * dv), store)
-    return o @ w[p + "o"].T
+    size = (m.get("mask") or {}).get("size")
+    o = attend(q, k, v, m["scale"], visible_keys(T, T, size), m.get("softcap"))
+    return stored(o.reshape(T, H * dv), store) @ w[p + "o"].T
 
 
 # --------------------------------------------------------------------------- latent attention
@@ -116,27 +130,25 @@ def latent_attention(h: torch.Tensor, w: dict, p: str, m: dict, eps: float,
     T = h.shape[0]
     H, d, r = int(m["heads"]), int(m["dim"]), int(m["rot_dim"])
     dv, rank = int(m["vdim"]), int(m["kv_rank"])
-    rot = m["rot"]
+    rot = m.get("rot")
     pos = torch.arange(T)
     q = stored(h @ w[p + "q"].T, store).view(T, H, d + r)
     down = stored(h @ w[p + "dkv"].T, store)
     c = stored(norm(down[:, :rank], w[p + "dkv.norm"], eps), store)
     k_rot = down[:, None, rank:rank + r]
     q_flat, q_rot = q[..., :d], q[..., d:]
-    q_rot = stored(rotate_pairs(q_rot, pos, int(rot["dims"]), rot["base"]), store)
-    k_rot = stored(rotate_pairs(k_rot, pos, int(rot["dims"]), rot["base"]), store)
+    if rot:
+        q_rot = rotate_pairs(q_rot, pos, int(rot["dims"]), rot["base"])
+        k_rot = rotate_pairs(k_rot, pos, int(rot["dims"]), rot["base"])
+    q_rot, k_rot = stored(q_rot, store), stored(k_rot, store)
     k_flat = stored(c @ w[p + "uk"].T, store).view(T, H, d)
     v = stored(c @ w[p + "uv"].T, store).view(T, H, dv)
-    s = (torch.einsum("thd,shd->hts", q_flat, k_flat)
-         + torch.einsum("thd,sd->hts", q_rot, k_rot[:, 0])) * float(m["scale"])
-    visible = pos[None, :] <= pos[:, None]
     size = (m.get("mask") or {}).get("size")
-    if size:
-        visible = visible & (pos[:, None] - pos[None, :] < int(size))
-    sink = w[p + "sink"].to(s.dtype) if (p + "sink") in w else None
-    a = softmax_rows(s, visible, sink)
-    o = stored(torch.einsum("hts,shd->thd", a, v).reshape(T, H * dv), store)
-    return o @ w[p + "o"].T
+    sink = w[p + "sink"].to(q.dtype) if (p + "sink") in w else None
+    # a head's key: its own read-out of the latent, then the part that all heads share
+    o = attend(torch.cat([q_flat, q_rot], -1), torch.cat([k_flat, k_rot.expand(T, H, r)], -1), v,
+               m["scale"], visible_keys(T, T, size), None, sink)
+    return stored(o.reshape(T, H * dv), store) @ w[p + "o"].T
 
 
 # ------------------------------------------------------------------------------------- wkv
@@ -213,3 +225,11 @@ def forward(config: dict, weights: dict, tokens, dtype: torch.dtype = torch.floa
     h = stored(norm(x, w["final.norm"], eps), store)
     logits = (h @ w["embed"].T) * float(config.get("logit_scale", 1.0))
     return capped(logits, config.get("logit_softcap")).to(torch.float32)
+
+
+def greedy(config: dict, weights: dict, prompt, n: int) -> list[int]:
+    """``n`` tokens by always taking the best one (the lowest index among equals)."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(forward(config, weights, toks)[-1].argmax()))
+    return toks[len(prompt):]

@@ -497,6 +497,80 @@ def rudorax_points(dtype, batch, prompt_len, steps, warmup, use_graphs=True, onl
     return out
 
 
+# (name, width, q heads, kv heads, head size, latent heads' plain / rotated / value size, latent rank,
+#  memory heads, their size, feed-forward, groups of four layers, vocabulary)
+BUZINEX_SIZES = [("w1024", 1024, 16, 4, 64, 64, 32, 64, 192, 16, 64, 4096, 2, 32000),
+                 ("w2048", 2048, 32, 8, 64, 64, 32, 64, 192, 32, 64, 8192, 2, 128256),
+                 ("w4096", 4096, 32, 8, 128, 128, 64, 128, 192, 64, 64, 14336, 1, 128256)]
+BUZINEX_WINDOW, BUZINEX_DECAY_RANK = 1024, 64
+
+
+def buzinex_points(dtype, batch, prompt_len, steps, warmup, use_graphs=True, only=None):
+    """Buzinex at a few sizes that resemble a real model's layers (groups of capped attention,
+    latent attention, a decaying matrix memory without a feed-forward, latent attention), beside
+    a Llama model of the same width, heads, feed-forward and number of layers that keeps every
+    key; random weights drawn on the device.  Per size and model: ms per decode step, its share
+    of the HBM roofline, tokens a second of a 2,048-token prefill and its share of the
+    matrix-core peak.  A Buzinex decode step has to read: every matrix once, the keys and values
+    of the attention layers, one latent row (``rot_dim + kv_rank``) per token of the window in
+    the latent layers, and every sequence's memories (read and written)."""
+    import torch
+    from kvforge_amd.config.presets import buzinex_stack
+
+    elem = 2 if dtype == "bfloat16" else 4
+    out = {}
+    for name, w, H, KV, d, ld, lr, lv, rank, Hm, dm, ff, groups, vocab in BUZINEX_SIZES:
+        if only and name not in only:
+            continue
+        layers = 4 * groups
+        llama = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": vocab,
+                 "hidden_size": w, "num_hidden_layers": layers, "num_attention_heads": H,
+                 "num_key_value_heads": KV, "head_dim": d, "intermediate_size": ff,
+                 "max_position_embeddings": CONTEXT_CAP, "rope_theta": 500000.0, "rope_scaling": None,
+                 "rms_norm_eps": 1e-5, "hidden_act": "silu", "tie_word_embeddings": True}
+        buz = buzinex_stack(vocab=vocab, width=w, groups=groups, heads=H, kv_heads=KV, dim=d, latent_dim=ld,
+                            rot_dim=lr, kv_rank=rank, window=BUZINEX_WINDOW, wkv_heads=Hm, wkv_dim=dm, ff=ff,
+                            max_positions=CONTEXT_CAP)
+        for layer in buz["layers"]:
+            if layer["type"] == "latent_attention":
+                layer["mixer"]["vdim"] = lv
+        attn = w * d * (2 * H + 2 * KV)
+        latent = w * (H * (ld + lr) + rank + lr) + H * (ld + lv) * rank + H * lv * w
+        memory = 5 * w * Hm * dm + BUZINEX_DECAY_RANK * (w + Hm * dm)
+        linear = groups * (attn + 2 * latent + memory + 3 * 3 * w * ff)
+        nums = {"llama": model_numbers(llama, layers),
+                "buzinex": {"linear_params": linear, "head_params": vocab * w,
+                            "kv_values_per_token": groups * 2 * KV * d, "attn_hd": H * d, "layers": groups}}
+        # what the latent layers add to a prompt's arithmetic: scores and sums over rot + rank and rank
+        state_bytes = groups * (Hm * dm * dm + w) * 4 * 2
+        for model, cfg in (("llama", llama), ("buzinex", buz)):
+            need = batch * (prompt_len + steps + warmup + early_tokens(batch, prompt_len) + 32)
+            engine = build_engine(cfg, dtype, batch, max(need, PREFILL_TOKENS + 64), use_graphs=use_graphs)
+            r = decode_run(engine, vocab, batch, prompt_len, steps, warmup)
+            s = prefill_run(engine, vocab, PREFILL_TOKENS, repeats=2)
+            if model == "llama":
+                read = decode_bytes(engine, nums[model], elem, batch, r["mean_ctx"])
+                flops = prefill_flops(nums[model], PREFILL_TOKENS)
+            else:
+                seen = min(r["mean_ctx"], BUZINEX_WINDOW)
+                read = ((linear + vocab * w) * elem
+                        + batch * (r["mean_ctx"] * nums[model]["kv_values_per_token"] * elem
+                                   + seen * 2 * groups * (lr + rank) * elem + state_bytes))
+                n = PREFILL_TOKENS
+                pairs = n * min(n, BUZINEX_WINDOW) - min(n, BUZINEX_WINDOW) ** 2 / 2.0     # (query, key) pairs under the window
+                flops = (prefill_flops(nums[model], n)
+                         + 2 * groups * 2.0 * pairs * H * (lr + 2 * rank)      # latent scores and sums
+                         + groups * n * Hm * 4.0 * dm * dm)                      # the memories' updates and reads
+            out[f"{name}_{model}"] = {
+                "decode_ms": round(r["ms_per_step"], 4), "decode_tok_s": round(r["tok_s"], 1),
+                "decode_hbm_frac": round(read / (r["seconds"] / steps) / 1e9 / HBM_PEAK_GBS, 4),
+                "prefill_tok_s": round(PREFILL_TOKENS / s, 1), "prefill_ms": round(s * 1e3, 3),
+                "prefill_frac": round(flops / s / MFMA_PEAK[dtype], 4)}
+            del engine
+            torch.cuda.empty_cache()
+    return out
+
+
 def model_numbers(cfg, layers_run):
     h, H, KV, d, I, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
                          cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"])
@@ -525,7 +599,8 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--decode-run-steps", type=int, default=None,
                     help="decode steps the device takes between two looks of the host (engine default: 8)")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products", "fogorax", "rudorax"], default="all",
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products", "fogorax", "rudorax", "buzinex"],
+                    default="all",
                     help="for profiles: only the decode steps at --batch, or only the prefill; "
                          "mixed: --batch requests with prompts of 128 to 4,096 tokens, chunked "
                          "prefill beside decode steps, --steps new tokens each; burst: the "
@@ -534,8 +609,9 @@ def main() -> int:
                          "products: the four matrix products of a layer alone at --batch rows "
                          "(launch to launch, so short ones show the host's time); fogorax: the "
                          "Fogorax design at a few layer sizes beside a Llama model of equal sizes; "
-                         "rudorax: the Rudorax design likewise (--sizes names some of them)")
-    ap.add_argument("--sizes", default="", help="with --phase rudorax: the sizes to run, with commas")
+                         "rudorax: the Rudorax design likewise (--sizes names some of them); "
+                         "buzinex: the Buzinex design likewise")
+    ap.add_argument("--sizes", default="", help="with --phase rudorax or buzinex: the sizes to run, with commas")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -565,6 +641,19 @@ def main() -> int:
                                                     "identity", "shared_ff", "layers", "vocab"), r[1:]))
                                     for r in RUDORAX_SIZES},
                           **rudorax_points(args.dtype, args.batch, args.prompt_len, steps,
+                                           min(args.warmup, 8), not args.no_graphs,
+                                           [x for x in args.sizes.split(",") if x] or None)}))
+        return 0
+    if args.phase == "buzinex":
+        steps = min(args.steps, 64)
+        print(json.dumps({"phase": "buzinex", "dtype": args.dtype, "batch": args.batch,
+                          "prompt_len": args.prompt_len, "steps": steps, "window": BUZINEX_WINDOW,
+                          "prefill_tokens": PREFILL_TOKENS,
+                          "sizes": {r[0]: dict(zip(("width", "heads", "kv_heads", "head_dim", "latent_dim",
+                                                    "latent_rot_dim", "latent_vdim", "kv_rank", "memory_heads",
+                                                    "memory_dim", "ff", "groups", "vocab"), r[1:]))
+                                    for r in BUZINEX_SIZES},
+                          **buzinex_points(args.dtype, args.batch, args.prompt_len, steps,
                                            min(args.warmup, 8), not args.no_graphs,
                                            [x for x in args.sizes.split(",") if x] or None)}))
         return 0

@@ -1374,15 +1374,47 @@ def tanh_cast(x: torch.Tensor, out: torch.Tensor) -> None:
     _ok(f(_tcode(out.dtype), x.data_ptr(), out.data_ptr(), x.numel(), _stream()), "tanh_cast")
 
 
+# Runs of at least WKV_MULTI_FROM tokens are cut into chunks of WKV_CHUNK tokens that go side by
+# side (three passes); shorter runs go token by token in one workgroup per head.
+WKV_CHUNK = 16
+WKV_MULTI_FROM = 64
+
+
+def wkv_multi_plan(q_lens, multi_from: int = WKV_MULTI_FROM) -> tuple[list[int], list[int]]:
+    """For the runs of at least ``multi_from`` tokens among ``q_lens`` (a step's runs in sequence
+    order): the flat rows ``(sequence, first token, tokens, 0)`` of their chunks and
+    ``(sequence, first chunk, chunks)`` of the runs, as ``wkv_scan(multi=...)`` wants them."""
+    chunks: list[int] = []
+    runs: list[int] = []
+    start = 0
+    for seq, q in enumerate(q_lens):
+        if q >= multi_from:
+            first = len(chunks) // 4
+            for t in range(0, q, WKV_CHUNK):
+                chunks += [seq, start + t, min(WKV_CHUNK, q - t), 0]
+            runs += [seq, first, len(chunks) // 4 - first]
+        start += q
+    return chunks, runs
+
+
+def wkv_multi_scratch(n_chunks: int, heads: int, dim: int) -> dict[str, tuple]:
+    """(shape, dtype) of the scratch tensors the passes over all chunks need, by name."""
+    return {"G": ((n_chunks, int(heads), int(dim), int(dim)), F32), "D": ((n_chunks, int(heads), int(dim)), F32)}
+
+
 def wkv_scan(rows: torch.Tensor, r_off: int, k_off: int, v_off: int, z: torch.Tensor, w0: torch.Tensor,
              u: torch.Tensor, cu_q: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Tensor,
-             state: torch.Tensor, out: torch.Tensor, n_seqs: int, heads: int, dim: int) -> None:
+             state: torch.Tensor, out: torch.Tensor, n_seqs: int, heads: int, dim: int,
+             multi: dict | None = None, short_runs: bool = True) -> None:
     """The recurrence ``o_j = sum_i r_i (S_ij + u_i k_i v_j)``, ``S_ij <- w_i S_ij + k_i v_j`` with
-    ``w = exp(-exp(z + w0))`` over every query run, token by token in fp32, from and to the
-    sequences' state slots (a run at position 0 starts from zeros whatever its slot holds; a
-    sequence without a slot starts from zeros and keeps nothing).  ``rows``: r, k, v of a
-    token ``[heads * dim]`` each at the given offsets of its row; ``z`` fp32 ``[n, >= heads *
-    dim]``; ``w0``, ``u`` fp32 ``[heads * dim]``; ``out`` fp32 ``[n, heads * dim]``."""
+    ``w = exp(-exp(z + w0))`` over every query run, in fp32, from and to the sequences' state
+    slots (a run at position 0 starts from zeros whatever its slot holds; a sequence without a
+    slot starts from zeros and keeps nothing).  ``rows``: r, k, v of a token ``[heads * dim]``
+    each at the given offsets of its row; ``z`` fp32 ``[n, >= heads * dim]``; ``w0``, ``u`` fp32
+    ``[heads * dim]``; ``out`` fp32 ``[n, heads * dim]``.  ``multi``: ``chunks`` and ``runs``
+    (int32 device tensors of ``wkv_multi_plan``'s rows) and the scratch ``G``, ``D``: those runs
+    go chunk by chunk side by side and the token-by-token kernel leaves them alone; it is not
+    launched at all with ``short_runs=False`` (the caller knows that no other run is there)."""
     n = rows.shape[0]
     H, dk = int(heads), int(dim)
     _check(rows, "rows", None, (n, None))
@@ -1401,11 +1433,27 @@ def wkv_scan(rows: torch.Tensor, r_off: int, k_off: int, v_off: int, z: torch.Te
         _check(t, name, I32, (None,))
     if cu_q.shape[0] < n_seqs + 1 or slot_ids.shape[0] < n_seqs or positions.shape[0] < n:
         raise KernelError("wkv_scan: batch arrays shorter than the batch")
-    f = _fn("wkv", "kvf_wkv_scan", [c_int] + [c_void_p] * 9 + [c_int] * 10 + [c_void_p])
-    _ok(f(_tcode(rows.dtype), rows.data_ptr(), z.data_ptr(), w0.data_ptr(), u.data_ptr(), cu_q.data_ptr(),
-          positions.data_ptr(), slot_ids.data_ptr(), state.data_ptr(), out.data_ptr(), int(n_seqs), H, dk,
-          state.shape[0], state.shape[1], rows.shape[1], int(r_off), int(k_off), int(v_off), z.shape[1],
-          _stream()), "wkv_scan")
+    common = (_tcode(rows.dtype), rows.data_ptr(), z.data_ptr(), w0.data_ptr(), u.data_ptr(), cu_q.data_ptr(),
+              positions.data_ptr(), slot_ids.data_ptr(), state.data_ptr(), out.data_ptr())
+    shape = (int(n_seqs), H, dk, state.shape[0], state.shape[1], rows.shape[1], int(r_off), int(k_off), int(v_off),
+             z.shape[1])
+    if short_runs or multi is None:
+        f = _fn("wkv", "kvf_wkv_scan", [c_int] + [c_void_p] * 9 + [c_int] * 11 + [c_void_p])
+        _ok(f(*common, *shape, WKV_MULTI_FROM if multi is not None else 0, _stream()), "wkv_scan")
+    if multi is None:
+        return
+    chunks, runs, G, D = multi["chunks"], multi["runs"], multi["G"], multi["D"]
+    _check(chunks, "chunks", I32, (None, 4))
+    _check(runs, "runs", I32, (None, 3))
+    nc = chunks.shape[0]
+    _check(G, "G", F32, (None, H, dk, dk))
+    _check(D, "D", F32, (None, H, dk))
+    if G.shape[0] < nc or D.shape[0] < nc:
+        raise KernelError("wkv_scan: scratch for fewer chunks than the plan has")
+    f = _fn("wkv", "kvf_wkv_chunks", [c_int] + [c_void_p] * 10 + [c_int, c_void_p, c_int, c_void_p, c_void_p]
+            + [c_int] * 10 + [c_void_p])
+    _ok(f(*common, chunks.data_ptr(), nc, runs.data_ptr(), runs.shape[0], G.data_ptr(), D.data_ptr(), *shape,
+          _stream()), "wkv_chunks")
 
 
 def wkv_out(heads_raw: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float,

@@ -104,6 +104,22 @@ class DecayMemory(Mixer):
     def held_tensors(self) -> list[torch.Tensor]:
         return [c for w in self._matrices() for c in ops.copies_of(w)] + self._small()
 
+    def _long_runs(self, step) -> dict | None:
+        """Chunk and run tables of this step's long runs (made once per step, shared by the layers
+        of the batch) and scratch from the step's workspace.  ``None`` when no run is that long."""
+        key = "wkv.long_runs"
+        plan = step.scratch.get(key)
+        if plan is None:
+            chunks, runs = ops.wkv_multi_plan(step.q_lens)
+            plan = (step.upload_ints(chunks).view(-1, 4), step.upload_ints(runs).view(-1, 3)) if chunks else ()
+            step.scratch[key] = plan
+        if not plan:
+            return None
+        out = {"chunks": plan[0], "runs": plan[1]}
+        for name, (shape, dtype) in ops.wkv_multi_scratch(plan[0].shape[0], self.H, self.dk).items():
+            out[name] = step.ws.buf("wkv_multi_" + name, shape, dtype)
+        return out
+
     def forward(self, x, step, layer: LayerState, residual) -> None:
         """``x``: normalised activations."""
         if layer.state is None:
@@ -125,8 +141,11 @@ class DecayMemory(Mixer):
         z = ws.buf("wkv_decay", (n, HD), torch.float32)
         ops.gemm(low_act, self.w_2, z)
         raw = ws.buf("wkv_raw", (n, HD), torch.float32)
+        # which kernels have work is known from the runs' lengths (all ones in a captured step of
+        # single tokens, so a replay launches what the capture launched)
         ops.wkv_scan(rows, 0, HD, 2 * HD, z, self.w0, self.u, step.cu_q, step.positions, step.slot_ids,
-                     layer.state, raw, step.n_seqs, H, dk)
+                     layer.state, raw, step.n_seqs, H, dk, multi=self._long_runs(step),
+                     short_runs=any(q < ops.WKV_MULTI_FROM for q in step.q_lens))
         heads = ws.buf("wkv_heads", (n, HD), act)
         ops.wkv_out(raw, rows[:, 3 * HD:], self.head_weight, self.norm_eps, heads, H, dk)
         add_product(step, heads, self.w_o, residual)

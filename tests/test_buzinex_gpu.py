@@ -260,6 +260,55 @@ def test_the_memory_over_runs_and_steps(dtype, H, dk):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,dk", [(2, 8), (3, 64), (2, 100), (1, 136), (1, 256)])
+def test_the_memory_over_long_runs_chunk_by_chunk(dtype, H, dk):
+    """Runs of 64 tokens and more are cut into chunks that go side by side; in one step with
+    them, short runs that go token by token.  A long run that goes on from what a short one left
+    and the other way round, a last chunk of one token and a full one, a slot that still holds
+    another's memory, a long run without a slot, and strong decays (whole chunks that forget
+    all that was before them)."""
+    HD = H * dk
+    lens = {"a": 235, "b": 70, "c": 129, "d": 5}
+    data = {r: (rand(n, 3 * HD, seed=i + dk).to(dtype), rand(n, HD, seed=i + 70, scale=2.0))
+            for i, (r, n) in enumerate(lens.items())}
+    data["c"][1][40:60] += 6.0                            # decays of exp(-exp(6 + ...)): nothing survives
+    w0, u = rand(HD, seed=9, scale=1.5) - 1.0, rand(HD, seed=10, scale=0.5)
+    want = {}
+    for r, (rows, z) in data.items():
+        x = rows.float()
+        decay = torch.exp(-torch.exp(z + w0)).view(-1, H, dk)
+        want[r] = plain.wkv_recurrence(x[:, :HD].reshape(-1, H, dk), x[:, HD:2 * HD].reshape(-1, H, dk),
+                                       x[:, 2 * HD:].reshape(-1, H, dk), decay, u.view(H, dk)).reshape(-1, HD)
+    state = torch.full((3, ops().wkv_state_floats(H, dk, 8)), 3.0, device=DEV)   # junk
+    slot = {"a": 2, "b": 0, "c": 1, "d": 1}
+    got = {r: [] for r in lens}
+    steps = ([("a", 0, 150), ("d", 0, 3)], [("a", 150, 153), ("b", 0, 70), ("d", 3, 5)],
+             [("c", 0, 64), ("a", 153, 170)], [("a", 170, 235), ("c", 64, 129)])
+    for step in steps:
+        rows = torch.cat([data[r][0][a:b] for r, a, b in step] + [data["b"][0][:65]]).to(DEV)
+        z = torch.cat([data[r][1][a:b] for r, a, b in step] + [data["b"][1][:65]]).to(DEV)
+        counts = [b - a for _, a, b in step] + [65]      # and a long run without a slot
+        cu = i32([0] + list(np.cumsum(counts)))
+        pos = torch.cat([torch.arange(a, b) for _, a, b in step] + [torch.arange(65)]).int().to(DEV)
+        chunks, runs = ops().wkv_multi_plan(counts)
+        assert len(runs) // 3 == sum(c >= 64 for c in counts) >= 2
+        nc = len(chunks) // 4
+        multi = {"chunks": i32(chunks).view(-1, 4), "runs": i32(runs).view(-1, 3),
+                 "G": torch.full((nc, H, dk, dk), 7.0, device=DEV), "D": torch.full((nc, H, dk), 7.0, device=DEV)}
+        out = torch.full((rows.shape[0], HD), 5.0, device=DEV)
+        ops().wkv_scan(rows, 0, HD, 2 * HD, z, w0.to(DEV), u.to(DEV), cu, pos,
+                       i32([slot[r] for r, _, _ in step] + [-1]), state, out, len(counts), H, dk, multi=multi,
+                       short_runs=any(c < 64 for c in counts))
+        off = 0
+        for (r, a, b) in step:
+            got[r].append(out[off:off + b - a].cpu())
+            off += b - a
+        torch.testing.assert_close(out[off:].cpu(), want["b"][:65], atol=2e-5 * float(want["b"].abs().max()), rtol=2e-4)
+    for r in lens:
+        torch.testing.assert_close(torch.cat(got[r]), want[r], atol=2e-5 * float(want[r].abs().max()), rtol=2e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,dk", [(3, 16), (2, 40), (1, 256)])
 def test_heads_normed_weighted_and_gated_and_the_decays_tanh(dtype, H, dk):
     n, eps = 5, 1e-3

@@ -11,9 +11,11 @@
 //                  the attention kernels' row [H q heads | k | v] of heads of d elements:
 //                  q head h = [q_r_h | (left for head_product) | 0], k = [k_r | norm(c) | 0],
 //                  v = [0 | norm(c) | 0]; the norm in fp32 with one rounding.
-//   head_product : out[n, h, :] = W[h] in[n, h, :] for per-head matrices W [H, O, I]
-//                  (fp32 multiply and add on the vector ALUs, tiles of 32 rows x 64 outputs
-//                  through LDS).
+//   head_product : out[n, h, :] = W[h] in[n, h, :] for per-head matrices W [H, O, I].  bf16 rows and
+//                  weights whose heads start on 16 bytes go to the matrix cores (a workgroup
+//                  per 64 rows x 64 outputs of a head, a wave per 16 outputs, operands straight
+//                  from memory, fp32 sums); everything else is fp32 multiply and add on the
+//                  vector ALUs, tiles of 32 rows x 64 outputs through LDS.
 #include "common.h"
 
 namespace {
@@ -107,6 +109,64 @@ __global__ __launch_bounds__(256) void head_product_kernel(const T* __restrict__
   }
 }
 
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+// v_mfma_f32_16x16x32_bf16 computes D[i][j] += sum_k A[i][k] B[j][k]; lane 16 c + r gives row r,
+// elements 8c..8c+7 of the step's 32 of either operand, and holds D[4 (l / 16) + v][l % 16].
+// A: 16 rows of the head's matrix (outputs), B: 16 rows of the input.  Grid (tiles of 64 rows,
+// tiles of 64 outputs, heads); wave w takes outputs 16w..16w+15 of the tile for all its rows, so a
+// weight fragment is loaded once for up to four row fragments.  I, in_head and ld_in are
+// multiples of 8 and both bases lie on 16 bytes (the host checks), so a fragment is one 16-byte
+// load that lies inside its row or is left zero.
+__global__ __launch_bounds__(256) void head_product_mfma_kernel(const bf16_t* __restrict__ in, int ld_in,
+                                                                int in_head, const bf16_t* __restrict__ W,
+                                                                bf16_t* __restrict__ out, int ld_out, int out_head,
+                                                                int N, int O, int I) {
+  const int n0 = blockIdx.x * 64, h = blockIdx.z;
+  const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
+  const int j = lane % 16, c = lane / 16;
+  const int o0 = blockIdx.y * 64 + wave * 16;
+  if (o0 >= O) return;
+  const int subs = min(4, (N - n0 + 15) / 16);
+  const bf16_t* wrow = o0 + j < O ? W + (static_cast<size_t>(h) * O + o0 + j) * I + 8 * c : nullptr;
+  const bf16_t* xr[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int n = n0 + 16 * r + j;
+    xr[r] = (r < subs && n < N) ? in + static_cast<size_t>(n) * ld_in + static_cast<size_t>(h) * in_head + 8 * c
+                                : nullptr;
+  }
+  f32x4 acc[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < I; k0 += 32) {
+    const bool inside = k0 + 8 * c + 8 <= I;
+    uint4 wf = make_uint4(0u, 0u, 0u, 0u);
+    if (wrow && inside) wf = *reinterpret_cast<const uint4*>(wrow + k0);
+    uint4 xf[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      xf[r] = make_uint4(0u, 0u, 0u, 0u);
+      if (xr[r] && inside) xf[r] = *reinterpret_cast<const uint4*>(xr[r] + k0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (r < subs)
+        acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf),
+                                                         __builtin_bit_cast(bf16x8, xf[r]), acc[r], 0, 0, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int n = n0 + 16 * r + j;
+    if (r >= subs || n >= N) continue;
+    bf16_t* o = out + static_cast<size_t>(n) * ld_out + static_cast<size_t>(h) * out_head + o0 + 4 * c;
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      if (o0 + 4 * c + v < O) Elem<bf16_t>::store(o + v, acc[r][v]);
+  }
+}
+
 template <typename T, typename TW>
 int head_product_launch(const void* in, int ld_in, int in_head, const void* W, void* out, int ld_out,
                         int out_head, int N, int H, int O, int I, hipStream_t s) {
@@ -143,6 +203,13 @@ KVF_EXPORT int kvf_head_product(int dtype, int wtype, const void* in, int ld_in,
   if (N <= 0) return 0;
   if (H <= 0 || O <= 0 || I <= 0 || H > 65535 || (O + HP_N - 1) / HP_N > 65535)
     return static_cast<int>(hipErrorInvalidValue);
+  if (dtype == 1 && wtype == 1 && I % 8 == 0 && in_head % 8 == 0 && ld_in % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0) {
+    const dim3 grid((N + 63) / 64, (O + 63) / 64, H);
+    hipLaunchKernelGGL(head_product_mfma_kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(in), ld_in, in_head,
+                       static_cast<const bf16_t*>(W), static_cast<bf16_t*>(out), ld_out, out_head, N, O, I);
+    return kvf_last_error();
+  }
   if (dtype == 0 && wtype == 0)
     return head_product_launch<float, float>(in, ld_in, in_head, W, out, ld_out, out_head, N, H, O, I, s);
   if (dtype == 1 && wtype == 1)

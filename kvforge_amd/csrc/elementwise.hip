@@ -1151,6 +1151,7 @@ KVF_EXPORT int kvf_token_side_bf16(TOKEN_SIDE_DECL) {
 //   settle_cast: x[m] += bias + owed[m] (either may be null); copy[m] = x[m] in T (copy may be null)
 //   side_gate:   g[m, j] = gelu_tanh(a[m, j]) * side[token[m], col0 + j]
 //   rms_add:     x[m] += y[m] * rsqrt(mean(y[m]^2) + eps) * w
+//   rms_add_norm: the same, and out[m] = x[m] * rsqrt(mean(x[m]^2) + eps2) * w2 of the new x
 template <typename T, typename D>
 __global__ void settle_cast_kernel(float* __restrict__ x, const float* __restrict__ bias,
                                    const D* __restrict__ owed, T* __restrict__ copy, int h, size_t total) {
@@ -1230,4 +1231,86 @@ KVF_EXPORT int kvf_rms_add(float* x, const float* y, const float* w, float eps, 
   if (m <= 0) return 0;
   hipLaunchKernelGGL(rms_add_kernel, dim3(m), dim3(256), 0, s, x, y, w, eps, h);
   return kvf_last_error();
+}
+
+// A sublayer's rows join the stream through their norm, and the next sublayer's input is the norm
+// of the sum: one pass over the row for both (a thread reads back only what it wrote itself).
+// EPT > 0: rows of at most 256 * EPT elements, which a thread then holds in registers: every load is
+// asked for before the first sum, and the row is read once.  EPT = 0: any width, three passes.
+template <typename T, int EPT>
+__global__ __launch_bounds__(256) void rms_add_norm_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                           const float* __restrict__ w, float eps,
+                                                           const float* __restrict__ w2, float eps2,
+                                                           T* __restrict__ out, int h) {
+  __shared__ float scratch[16], scratch2[16];
+  const int m = blockIdx.x;
+  float* xr = x + static_cast<size_t>(m) * h;
+  const float* yr = y + static_cast<size_t>(m) * h;
+  T* o = out + static_cast<size_t>(m) * h;
+  if (EPT > 0) {
+    constexpr int N = EPT > 0 ? EPT : 1;
+    float yv[N], xv[N], wv[N], w2v[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const int i = k * 256 + threadIdx.x;
+      const bool ok = i < h;
+      yv[k] = ok ? yr[i] : 0.f;
+      xv[k] = ok ? xr[i] : 0.f;
+      wv[k] = ok ? w[i] : 0.f;
+      w2v[k] = ok ? w2[i] : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < N; ++k) ss = fmaf(yv[k], yv[k], ss);
+    const float r = rsqrtf(block_sum(ss, scratch) / static_cast<float>(h) + eps);
+    float ss2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      xv[k] = fmaf(yv[k] * r, wv[k], xv[k]);
+      ss2 = fmaf(xv[k], xv[k], ss2);
+    }
+    const float r2 = rsqrtf(block_sum(ss2, scratch2) / static_cast<float>(h) + eps2);
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const int i = k * 256 + threadIdx.x;
+      if (i < h) {
+        xr[i] = xv[k];
+        Elem<T>::store(o + i, xv[k] * r2 * w2v[k]);
+      }
+    }
+    return;
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) ss = fmaf(yr[i], yr[i], ss);
+  const float r = rsqrtf(block_sum(ss, scratch) / static_cast<float>(h) + eps);
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    const float v = fmaf(yr[i] * r, w[i], xr[i]);
+    xr[i] = v;
+    ss2 = fmaf(v, v, ss2);
+  }
+  const float r2 = rsqrtf(block_sum(ss2, scratch2) / static_cast<float>(h) + eps2);
+  for (int i = threadIdx.x; i < h; i += blockDim.x) Elem<T>::store(o + i, xr[i] * r2 * w2[i]);
+}
+template <typename T>
+static int rms_add_norm_launch(float* x, const float* y, const float* w, float eps, const float* w2, float eps2,
+                               void* out, int m, int h, hipStream_t s) {
+  if (h <= 256 * 4)
+    hipLaunchKernelGGL((rms_add_norm_kernel<T, 4>), dim3(m), dim3(256), 0, s, x, y, w, eps, w2, eps2,
+                       static_cast<T*>(out), h);
+  else if (h <= 256 * 16)
+    hipLaunchKernelGGL((rms_add_norm_kernel<T, 16>), dim3(m), dim3(256), 0, s, x, y, w, eps, w2, eps2,
+                       static_cast<T*>(out), h);
+  else
+    hipLaunchKernelGGL((rms_add_norm_kernel<T, 0>), dim3(m), dim3(256), 0, s, x, y, w, eps, w2, eps2,
+                       static_cast<T*>(out), h);
+  return kvf_last_error();
+}
+// dtype of out: 0 = fp32, 1 = bf16
+KVF_EXPORT int kvf_rms_add_norm(int dtype, float* x, const float* y, const float* w, float eps, const float* w2,
+                                float eps2, void* out, int m, int h, hipStream_t s) {
+  if (m <= 0) return 0;
+  if (dtype == 0) return rms_add_norm_launch<float>(x, y, w, eps, w2, eps2, out, m, h, s);
+  if (dtype == 1) return rms_add_norm_launch<bf16_t>(x, y, w, eps, w2, eps2, out, m, h, s);
+  return static_cast<int>(hipErrorInvalidValue);
 }

@@ -11,7 +11,8 @@
 //              the slot after it has read the slot (no other workgroup touches it).
 //   wkv_scan : token by token.  A workgroup per (64 value columns, head, sequence); a thread
 //              owns one value column of up to 64 key rows of S in registers (a wave per 64 key
-//              rows); r, k, w of a stage of tokens go through LDS.  Everything is fp32; the
+//              rows); r, k, w of a stage of tokens go through LDS, from where lane l takes row
+//              l's and the wave passes them round lane by lane.  Everything is fp32; the
 //              order of every sum is fixed by the shapes, so a token's output does not depend
 //              on how its sequence was cut into runs.
 //   wkv_chunks : long runs, cut into chunks of 16 tokens that go side by side.  Over a chunk that
@@ -143,28 +144,42 @@ __global__ __launch_bounds__(256) void wkv_scan_kernel(const T* __restrict__ row
     if (MODE == CHUNK_STATE && static_cast<int>(threadIdx.x) < dk)
       for (int t = 0; t < cnt; ++t) decayed *= ws[t * dk + threadIdx.x];
     // the bonus of a token, sum_i r_i u_i k_i: a wave a token, lanes side by side along i
-    for (int t = part; MODE != CHUNK_STATE && t < cnt; t += parts) {
+    for (int t = part; MODE != CHUNK_STATE && parts > 1 && t < cnt; t += parts) {
       float b = 0.f;
       for (int e = lane; e < dk; e += KVF_WAVE) b = fmaf(rs[t * dk + e] * uh[e], ks[t * dk + e], b);
       b = wave_sum(b);
       if (lane == 0) bonus[t] = b;
     }
+    // lane l of a wave takes r, k, w of the wave's row l out of LDS once per token; every row's
+    // three numbers then reach all lanes as scalars (v_readlane), not as 64 broadcast reads
+    const int my_row = row0 + lane;
+    const bool row_ok = lane < ROWS && my_row < dk;
+    const float ul = row_ok ? uh[my_row] : 0.f;
     for (int t = 0; t < cnt; ++t) {
       const float v = vs[t * KVF_WAVE + lane];
-      const float* r = rs + t * dk + row0;
-      const float* k = ks + t * dk + row0;
-      const float* w = ws + t * dk + row0;
+      const int rl = row_ok ? __float_as_int(rs[t * dk + my_row]) : 0;
+      const int kl = row_ok ? __float_as_int(ks[t * dk + my_row]) : 0;
+      const int wl = row_ok ? __float_as_int(ws[t * dk + my_row]) : 0;   // rows past dk: S stays 0
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < ROWS; ++i) {
-        if (row0 + i < dk) {
-          acc = fmaf(r[i], S[i], acc);
-          S[i] = fmaf(w[i], S[i], k[i] * v);
-        }
+        const float ri = __int_as_float(__builtin_amdgcn_readlane(rl, i));
+        const float ki = __int_as_float(__builtin_amdgcn_readlane(kl, i));
+        const float wi = __int_as_float(__builtin_amdgcn_readlane(wl, i));
+        acc = fmaf(ri, S[i], acc);
+        S[i] = fmaf(wi, S[i], ki * v);
       }
-      if (MODE != CHUNK_STATE) psum[(t * parts + part) * KVF_WAVE + lane] = acc;
+      if (MODE == CHUNK_STATE) continue;
+      if (parts == 1) {
+        // one wave has all rows: the token's output is complete here (the bonus summed over the
+        // lanes' own rows, in the order the wider case sums it)
+        const float b = wave_sum(__int_as_float(rl) * ul * __int_as_float(kl));
+        if (col_ok) out[(static_cast<size_t>(tb + t) * a.H + head) * dk + col] = fmaf(v, b, acc);
+      } else {
+        psum[(t * parts + part) * KVF_WAVE + lane] = acc;
+      }
     }
-    if (MODE == CHUNK_STATE) continue;     // (the next stage starts with a barrier)
+    if (MODE == CHUNK_STATE || parts == 1) continue;     // (the next stage starts with a barrier)
     __syncthreads();
     for (int i = threadIdx.x; i < cnt * KVF_WAVE; i += blockDim.x) {
       const int t = i / KVF_WAVE, l = i % KVF_WAVE, c = blockIdx.x * KVF_WAVE + l;

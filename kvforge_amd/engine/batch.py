@@ -232,18 +232,32 @@ class Step:
         """The product owed to ``residual``, for a norm kernel that adds it itself."""
         if self.owed is None:
             return None
-        if self.owed[0] is not residual:
+        if self.owed[0] is not residual or len(self.owed) != 2:
             self.settle()
             return None
         product = self.owed[1]
         self.owed = None
         return product
 
+    def take_owed_normed(self, residual: torch.Tensor) -> tuple | None:
+        """``(rows, weight, eps)`` if what is owed to ``residual`` is the RMS norm of fp32 rows (a
+        sublayer's output that joins the stream through a norm of its own), for a kernel that
+        adds it itself; ``None`` otherwise (whatever else is owed stays owed)."""
+        if self.owed is None or self.owed[0] is not residual or len(self.owed) != 4:
+            return None
+        owed = self.owed[1:]
+        self.owed = None
+        return owed
+
     def settle(self) -> None:
-        """Add what is owed to the residual stream now."""
+        """Add what is owed to the residual stream now: ``(stream, rows)``, or ``(stream, rows,
+        weight, eps)`` for rows that join through their RMS norm."""
         if self.owed is not None:
             from kvforge_amd.kernels import ops
-            ops.add_rows(*self.owed)
+            if len(self.owed) == 4:
+                ops.rms_add(*self.owed)
+            else:
+                ops.add_rows(*self.owed)
             self.owed = None
 
 

@@ -369,6 +369,21 @@ def rms_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) 
         "rms_add")
 
 
+def rms_add_norm(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, weight2: torch.Tensor,
+                 eps2: float, out: torch.Tensor) -> None:
+    """``rms_add`` and the norm of the sum in one pass: ``x[m] += y[m] * rsqrt(mean(y[m]^2) + eps) *
+    weight``, then ``out[m] = x[m] * rsqrt(mean(x[m]^2) + eps2) * weight2``; both weights fp32."""
+    _check(x, "x", F32, (None, None))
+    _check(y, "y", F32, tuple(x.shape))
+    _check(weight, "weight", F32, (x.shape[1],))
+    _check(weight2, "weight2", F32, (x.shape[1],))
+    _check(out, "out", None, tuple(x.shape))
+    f = _fn("elementwise", "kvf_rms_add_norm", [c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float,
+                                                c_void_p, c_int, c_int, c_void_p])
+    _ok(f(_tcode(out.dtype), x.data_ptr(), y.data_ptr(), weight.data_ptr(), float(eps), weight2.data_ptr(),
+          float(eps2), out.data_ptr(), x.shape[0], x.shape[1], _stream()), "rms_add_norm")
+
+
 # ------------------------------------------------------------------------------ SwiGLU gate
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, paired: bool = False) -> None:
     """``out[:, i] = silu(gate_i) * up_i`` where the input row holds gate at ``i`` and up at

@@ -175,21 +175,39 @@ class SandwichBlock(Block):
     def forward(self, residual, step, layer: LayerState) -> None:
         shape = tuple(residual.shape)
         x = step.ws.buf("normed", shape, step.act_dtype)
-        self.pre.forward(residual, x, add=step.take_owed(residual))
+        self._norm_in(self.pre, residual, x, step)
         branch = step.ws.buf("sublayer_out", shape, torch.float32)
         step.fresh = branch
         self.mixer.forward(x, step, layer, branch)
         self._join(residual, branch, self.post, step)
         if self.ffn is None:
             return
-        self.ffn_pre.forward(residual, x)
+        self._norm_in(self.ffn_pre, residual, x, step)
         step.fresh = branch
         self.ffn.forward(x, step, branch)
         self._join(residual, branch, self.ffn_post, step)
 
     @staticmethod
     def _join(residual, branch, post: Norm, step) -> None:
+        """The sublayer's rows stay owed to the stream, through their norm, until the stream is
+        read next: by the norm in front of the next sublayer (one kernel for the sum and that
+        norm), or by whoever settles the step."""
         if step.fresh is branch:
             raise RuntimeError("a sublayer of a sandwich block must end in parts.base.add_product")
         step.settle()
-        post.add_to(residual, branch)
+        weight = post.fp32_weight() if hasattr(post, "fp32_weight") else None
+        if weight is None:
+            post.add_to(residual, branch)
+        else:
+            step.owed = (residual, branch, weight, post.eps)
+
+    @staticmethod
+    def _norm_in(norm: Norm, residual, x, step) -> None:
+        owed = step.take_owed_normed(residual)
+        weight = norm.fp32_weight() if hasattr(norm, "fp32_weight") else None
+        if owed is not None and weight is not None:
+            ops.rms_add_norm(residual, owed[0], owed[1], owed[2], weight, norm.eps, x)
+            return
+        if owed is not None:
+            ops.rms_add(residual, *owed)
+        norm.forward(residual, x, add=step.take_owed(residual))

@@ -43,6 +43,13 @@ class RMSNorm(Norm):
             self.weight = self.weight.float()    # the kernel multiplies by an fp32 vector
         ops.rms_add(stream, y, self.weight, self.eps)
 
+    def fp32_weight(self) -> torch.Tensor | None:
+        """The weight vector as the fused kernels take it (fp32, as it multiplies), or ``None``
+        for a norm that is not a plain ``x * rsqrt(mean(x^2) + eps) * weight`` with such a weight."""
+        if type(self).forward is not RMSNorm.forward or self.weight is None or self.weight.dtype != torch.float32:
+            return None
+        return self.weight
+
     def foldable_into(self, matrix: torch.Tensor) -> bool:
         """Whether this norm's weight may be multiplied into the columns of a bf16 matrix: only
         when it is itself held in bf16 (a weight stored in 32-bit stays a 32-bit multiply)."""

@@ -59,6 +59,21 @@ def test_a_sublayers_rows_are_normed_and_added_to_the_stream(h):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("h", [36, 100, 1024, 1030, 2500, 4096, 5000])
+def test_the_sum_and_the_next_sublayers_norm_in_one_pass(dtype, h):
+    x, y = rand(7, h, seed=h, scale=3.0), rand(7, h, seed=h + 1, scale=0.01)
+    w, w2 = 1.0 + rand(h, seed=2, scale=0.3), 1.0 + rand(h, seed=3, scale=0.3)
+    y[3] = 0.0
+    x[5] = 0.0                                          # the stream is all the sublayer's here
+    dev = x.clone().to(DEV)
+    out = torch.zeros(7, h, dtype=dtype, device=DEV)
+    ops().rms_add_norm(dev, y.to(DEV), w.to(DEV), 1e-5, w2.to(DEV), 1e-3, out)
+    stream = x + plain.norm(y, w, 1e-5)
+    torch.testing.assert_close(dev.cpu(), stream, atol=3e-5, rtol=3e-5)
+    torch.testing.assert_close(out.float().cpu(), plain.norm(stream, w2, 1e-3), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,KV,dk,d,coef,every", [(4, 2, 16, 16, 0.5, 4), (3, 1, 24, 32, 0.25, 1), (8, 1, 64, 64, 2.0, 7),
                                                   (5, 5, 7, 16, 0.1, 1000), (2, 1, 256, 256, 1.0, 64)])
 def test_head_norm_and_query_temperature_without_rotation(dtype, H, KV, dk, d, coef, every):

@@ -359,7 +359,7 @@ def shape_a():
     return make_config(vocab=211, width=72, layers=[("attention", att, 88), ("latent_attention", lat, 40),
                                                     ("wkv", rec, None), ("latent_attention", lat, None),
                                                     ("attention", att, None), ("wkv", rec, 56)],
-                       embedding_scale=6.5, logit_scale=0.3, logit_softcap=20.0, eps=1e-5, max_positions=512)
+                       embedding_scale=6.5, logit_scale=0.3, logit_softcap=20.0, eps=1e-5, max_positions=2048)
 
 
 def shape_b():
@@ -390,7 +390,20 @@ def shape_c():
                        embedding_scale=11.3, logit_scale=0.09, logit_softcap=30.0, eps=1e-6, max_positions=512)
 
 
-SHAPE = {"a": shape_a, "b": shape_b, "c": shape_c}
+def shape_d():
+    """Layers wide enough for the kernels that serving a real model takes: heads of 64 on the
+    matrix cores, a latent row of 32 + 160 elements, `head_product` on the matrix cores, a
+    feed-forward deep enough for a down projection cut in two halves of K, memory heads of one
+    wave each, a vocabulary that ends inside a group of 16 columns."""
+    att = dict(heads=6, kv_heads=2, dim=64, vdim=64, scale=0.125, softcap=25.0, q_temp=(0.35, 32))
+    lat = dict(heads=6, dim=64, rot_dim=32, vdim=64, kv_rank=160, scale=0.1, window=50, base=100000.0)
+    rec = dict(heads=6, dim=64, decay_rank=32)
+    return make_config(vocab=1000, width=384, layers=[("latent_attention", lat, 4096), ("wkv", rec, None),
+                                                      ("attention", att, 1024), ("latent_attention", lat, None)],
+                       embedding_scale=19.6, logit_scale=0.05, logit_softcap=25.0, eps=1e-5, max_positions=2048)
+
+
+SHAPE = {"a": shape_a, "b": shape_b, "c": shape_c, "d": shape_d}
 
 
 def liven(folder: str) -> None:
@@ -546,6 +559,20 @@ def test_unequal_requests_in_one_batch_against_each_alone(tmp_path_factory, name
         truth, plain_runs = plain_logits(cfg, w, t, dtype)
         close_to_truth(together[r], alone, [p + (alone - truth) for p in plain_runs], dtype,
                        f"{name} {r} against itself alone")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["a", "d"])
+def test_a_prompt_of_a_thousand_tokens(tmp_path_factory, name, dtype):
+    """Dozens of chunks of the memory side by side, the window over many pages, the temperature
+    over many steps: whole, in large and small portions, and its last tokens one by one."""
+    folder, cfg, w = model_folder(tmp_path_factory, name, dtype)
+    runner = make_runner(folder, dtype, block_size=16, num_blocks=80, tokens=1200)
+    toks = prompts_for(cfg, [1100], 11)["r0"]
+    for plan in ([[("r0", 0, 1100)]], in_portions("r0", 1100, (300, 64, 65, 7, 129, 2)),
+                 [[("r0", 0, 1050)]] + [[("r0", i, i + 1)] for i in range(1050, 1100)]):
+        got = replay(runner, {"r0": toks}, plan)["r0"]
+        check(got, cfg, w, toks, dtype, f"{name}, {len(plan)} steps")
 
 
 def marked_model(tmp_path, dtype, kind, window=None):

@@ -842,3 +842,36 @@ def test_trace_replay_in_a_process_of_its_own(tmp_path_factory, tmp_path, dtype)
         runs = [torch.stack([want[rid.split("#")[0]][1][k][pos] for rid, pos in rows])
                 for k in range(len(next(iter(want.values()))[1]))]
         close_to_truth(got, truth, runs, td, f"step {sid}")
+
+
+@pytest.mark.parametrize("kind", ["attention", "latent_attention", "wkv"])
+def test_trace_replay_of_a_model_of_one_kind(tmp_path, kind):
+    """A model with pages and no state slots, with windowed pages alone, and with state slots and
+    no pages at all, through ``bin/trace_run`` in bfloat16."""
+    mixer = {"attention": dict(heads=4, kv_heads=1, dim=32, vdim=16, scale=0.2, softcap=9.0, q_temp=(0.7, 24)),
+             "latent_attention": dict(heads=2, dim=24, rot_dim=8, vdim=40, kv_rank=56, scale=0.2, window=70,
+                                      base=30000.0),
+             "wkv": dict(heads=4, dim=32, decay_rank=5)}[kind]
+    cfg = make_config(vocab=150, width=80, layers=[(kind, mixer, 48), (kind, mixer, None)], embedding_scale=9.0,
+                      logit_scale=0.4, logit_softcap=12.0, eps=1e-5, max_positions=1024)
+    folder = str(tmp_path / "m")
+    kvforge_amd.write_random_model(folder, cfg, seed=3, dtype="bfloat16")
+    liven(folder)
+    w = load_file(os.path.join(folder, "model.safetensors"))
+    prompts = prompts_for(cfg, [90, 150, 33, 71], 12)
+    tb = ru.TraceBuilder()
+    for rid, toks in prompts.items():
+        ru.decode_tail(tb, f"{rid}#d", toks)
+        ru.portions(tb, f"{rid}#p", toks)
+    ru.mixed(tb, {f"{rid}#m": toks for rid, toks in prompts.items()}, 4)
+    out = str(tmp_path / "out")
+    ru.run_trace(folder, "bfloat16", tb, out)
+    want = {rid: plain_logits(cfg, w, toks, torch.bfloat16) for rid, toks in prompts.items()}
+    for sid, rows in enumerate(tb.expect):
+        if not rows:
+            continue
+        got = torch.from_numpy(np.fromfile(os.path.join(out, f"{sid}.f32"), dtype="<f4").reshape(-1, cfg["vocab"]).copy())
+        truth = torch.stack([want[rid.split("#")[0]][0][pos] for rid, pos in rows])
+        runs = [torch.stack([want[rid.split("#")[0]][1][k][pos] for rid, pos in rows]) for k in range(7)]
+        close_to_truth(got, truth, runs, torch.bfloat16, f"{kind}, step {sid}")
+

@@ -112,6 +112,21 @@ __global__ __launch_bounds__(256) void head_product_kernel(const T* __restrict__
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+// a lane's four neighbouring outputs: one 8-byte store where the output rows allow it (`wide`:
+// every head's outputs start on 8 bytes) and all four lie inside the head, else one by one
+__device__ __forceinline__ void store4(bf16_t* o, const f32x4& a, int left, bool wide) {
+  if (wide && left >= 4) {
+    uint2 p;
+    p.x = static_cast<unsigned>(f32_to_bf16(a[0])) | (static_cast<unsigned>(f32_to_bf16(a[1])) << 16);
+    p.y = static_cast<unsigned>(f32_to_bf16(a[2])) | (static_cast<unsigned>(f32_to_bf16(a[3])) << 16);
+    *reinterpret_cast<uint2*>(o) = p;
+    return;
+  }
+#pragma unroll
+  for (int v = 0; v < 4; ++v)
+    if (v < left) Elem<bf16_t>::store(o + v, a[v]);
+}
+
 // v_mfma_f32_16x16x32_bf16 computes D[i][j] += sum_k A[i][k] B[j][k]; lane 16 c + r gives row r,
 // elements 8c..8c+7 of the step's 32 of either operand, and holds D[4 (l / 16) + v][l % 16].
 // A: 16 rows of the head's matrix (outputs), B: 16 rows of the input.  Grid (tiles of 64 rows,
@@ -122,7 +137,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 __global__ __launch_bounds__(256) void head_product_mfma_kernel(const bf16_t* __restrict__ in, int ld_in,
                                                                 int in_head, const bf16_t* __restrict__ W,
                                                                 bf16_t* __restrict__ out, int ld_out, int out_head,
-                                                                int N, int O, int I) {
+                                                                int N, int O, int I, bool wide) {
   const int n0 = blockIdx.x * 64, h = blockIdx.z;
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
   const int j = lane % 16, c = lane / 16;
@@ -161,9 +176,63 @@ __global__ __launch_bounds__(256) void head_product_mfma_kernel(const bf16_t* __
     const int n = n0 + 16 * r + j;
     if (r >= subs || n >= N) continue;
     bf16_t* o = out + static_cast<size_t>(n) * ld_out + static_cast<size_t>(h) * out_head + o0 + 4 * c;
+    store4(o, acc[r], O - (o0 + 4 * c), wide);
+  }
+}
+
+// The same for many rows: a workgroup takes 64 rows of a head and ALL its outputs.  The rows'
+// fragments (KS steps of 32 elements cover I) are loaded once and stay in registers while the
+// wave goes through its groups of 16 outputs (w, w + 4, ...), so a row is read once per wave
+// and not once per wave and output tile.  Sums run over the steps in the same order as above.
+template <int KS>
+__global__ __launch_bounds__(256) void head_product_mfma_rows_kernel(const bf16_t* __restrict__ in, int ld_in,
+                                                                     int in_head, const bf16_t* __restrict__ W,
+                                                                     bf16_t* __restrict__ out, int ld_out,
+                                                                     int out_head, int N, int O, int I, bool wide) {
+  const int n0 = blockIdx.x * 64, h = blockIdx.y;
+  const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
+  const int j = lane % 16, c = lane / 16;
+  const int subs = min(4, (N - n0 + 15) / 16);
+  uint4 xf[KS][4];
 #pragma unroll
-    for (int v = 0; v < 4; ++v)
-      if (o0 + 4 * c + v < O) Elem<bf16_t>::store(o + v, acc[r][v]);
+  for (int r = 0; r < 4; ++r) {
+    const int n = n0 + 16 * r + j;
+    const bf16_t* x = (r < subs && n < N)
+                          ? in + static_cast<size_t>(n) * ld_in + static_cast<size_t>(h) * in_head + 8 * c
+                          : nullptr;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      xf[s][r] = make_uint4(0u, 0u, 0u, 0u);
+      if (x && 32 * s + 8 * c + 8 <= I) xf[s][r] = *reinterpret_cast<const uint4*>(x + 32 * s);
+    }
+  }
+  const int groups = (O + 15) / 16;
+  for (int g = wave; g < groups; g += 4) {
+    const int o0 = 16 * g;
+    const bf16_t* wrow = o0 + j < O ? W + (static_cast<size_t>(h) * O + o0 + j) * I + 8 * c : nullptr;
+    uint4 wf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      wf[s] = make_uint4(0u, 0u, 0u, 0u);
+      if (wrow && 32 * s + 8 * c + 8 <= I) wf[s] = *reinterpret_cast<const uint4*>(wrow + 32 * s);
+    }
+    f32x4 acc[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (r < subs)
+          acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf[s]),
+                                                           __builtin_bit_cast(bf16x8, xf[s][r]), acc[r], 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = n0 + 16 * r + j;
+      if (r >= subs || n >= N) continue;
+      bf16_t* o = out + static_cast<size_t>(n) * ld_out + static_cast<size_t>(h) * out_head + o0 + 4 * c;
+      store4(o, acc[r], O - (o0 + 4 * c), wide);
+    }
   }
 }
 
@@ -205,9 +274,28 @@ KVF_EXPORT int kvf_head_product(int dtype, int wtype, const void* in, int ld_in,
     return static_cast<int>(hipErrorInvalidValue);
   if (dtype == 1 && wtype == 1 && I % 8 == 0 && in_head % 8 == 0 && ld_in % 8 == 0 &&
       reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0) {
-    const dim3 grid((N + 63) / 64, (O + 63) / 64, H);
-    hipLaunchKernelGGL(head_product_mfma_kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(in), ld_in, in_head,
-                       static_cast<const bf16_t*>(W), static_cast<bf16_t*>(out), ld_out, out_head, N, O, I);
+    const bf16_t* x = static_cast<const bf16_t*>(in);
+    const bf16_t* w = static_cast<const bf16_t*>(W);
+    bf16_t* y = static_cast<bf16_t*>(out);
+    const dim3 rows((N + 63) / 64, H);
+    const bool wide = ld_out % 4 == 0 && out_head % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0;
+    if (N < 256 || I > 256) {   // few rows: more workgroups, each with one tile of outputs
+      const dim3 grid((N + 63) / 64, (O + 63) / 64, H);
+      hipLaunchKernelGGL(head_product_mfma_kernel, grid, dim3(256), 0, s, x, ld_in, in_head, w, y, ld_out, out_head, N,
+                         O, I, wide);
+    } else if (I <= 64) {
+      hipLaunchKernelGGL(head_product_mfma_rows_kernel<2>, rows, dim3(256), 0, s, x, ld_in, in_head, w, y, ld_out,
+                         out_head, N, O, I, wide);
+    } else if (I <= 128) {
+      hipLaunchKernelGGL(head_product_mfma_rows_kernel<4>, rows, dim3(256), 0, s, x, ld_in, in_head, w, y, ld_out,
+                         out_head, N, O, I, wide);
+    } else if (I <= 192) {
+      hipLaunchKernelGGL(head_product_mfma_rows_kernel<6>, rows, dim3(256), 0, s, x, ld_in, in_head, w, y, ld_out,
+                         out_head, N, O, I, wide);
+    } else {
+      hipLaunchKernelGGL(head_product_mfma_rows_kernel<8>, rows, dim3(256), 0, s, x, ld_in, in_head, w, y, ld_out,
+                         out_head, N, O, I, wide);
+    }
     return kvf_last_error();
   }
   if (dtype == 0 && wtype == 0)

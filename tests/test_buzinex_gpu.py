@@ -174,28 +174,30 @@ def test_a_projected_row_becomes_one_key_and_per_head_queries(dtype, H, dim, rot
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("n", [1, 33, 100, 200])
+@pytest.mark.parametrize("n", [1, 33, 100, 200, 257, 330])
 @pytest.mark.parametrize("lead", [2, 8])
 @pytest.mark.parametrize("H,O,I,in_head,out_head", [(4, 24, 16, 24, 32), (3, 36, 20, 32, 48), (1, 100, 70, 70, 100),
                                                     (5, 8, 130, 130, 8), (2, 192, 128, 192, 256), (3, 72, 40, 48, 80),
-                                                    (2, 130, 200, 200, 136)])
+                                                    (2, 130, 200, 200, 136), (2, 40, 256, 256, 40), (1, 24, 264, 264, 32)])
 def test_a_matrix_per_head(dtype, n, lead, H, O, I, in_head, out_head):
     """Rows in which a head starts every ``in_head`` elements and uses ``I`` of them; outputs
     written into wider rows, the columns between them left alone.  Rows that start ``lead``
     elements into wider ones: with 8 (and sizes that are multiples of 8) bfloat16 heads start on
-    16 bytes, which is what the matrix-core kernel takes; the others go through the plain one."""
+    16 bytes, which is what the matrix-core kernels take (one for few rows, one that keeps the rows
+    in registers from 256 rows on); the others go through the plain one."""
     x = rand(n, H * in_head + 8, seed=O).to(dtype)
     w = rand(H, O, I, seed=I, scale=I ** -0.5).to(dtype)
-    out = torch.full((n, H * out_head + 3), 7.0, dtype=dtype, device=DEV)
-    ops().head_product(x.to(DEV)[:, lead:], in_head, w.to(DEV), out[:, 1:], out_head)
+    pad = 1 if lead == 2 else 4              # (with 4, output rows whose heads start on 8 bytes)
+    out = torch.full((n, H * out_head + 2 * pad), 7.0, dtype=dtype, device=DEV)
+    ops().head_product(x.to(DEV)[:, lead:], in_head, w.to(DEV), out[:, pad:], out_head)
     xs = torch.stack([x.float()[:, lead + h * in_head:lead + h * in_head + I] for h in range(H)], 1)
     want = torch.einsum("nhi,hoi->nho", xs, w.float())
     got = out.float().cpu()
     for h in range(H):
-        torch.testing.assert_close(got[:, 1 + h * out_head:1 + h * out_head + O], want[:, h], **tol(dtype))
-    assert float(got[:, 0].min()) == 7.0
+        torch.testing.assert_close(got[:, pad + h * out_head:pad + h * out_head + O], want[:, h], **tol(dtype))
+    assert float(got[:, :pad].min()) == 7.0 and float(got[:, pad + (H - 1) * out_head + O:].min()) == 7.0
     if out_head > O:
-        assert float((got[:, 1 + O:1 + out_head] - 7.0).abs().max()) == 0.0
+        assert float((got[:, pad + O:pad + out_head] - 7.0).abs().max()) == 0.0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -24,6 +24,15 @@
 namespace {
 constexpr int ITEM_ROWS = 64;   // rows per work item: four waves of 16
 
+// The first key a query at position `pos` sees: with a window w > 0 the key w - 1 before it, with
+// chunks (window < 0, chunks of -window positions counted from position 0) the first key of its
+// own chunk.  It does not fall as `pos` grows.
+__device__ __forceinline__ int first_seen(int window, int pos) {
+  if (window > 0) return pos - window + 1 > 0 ? pos - window + 1 : 0;
+  if (window < 0) return pos - pos % (-window);
+  return 0;
+}
+
 struct AttnArgs {
   int H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs;
   int keep;  // with a window: the first `keep` keys of a sequence stay visible
@@ -104,13 +113,13 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
   if (last >= rows_total) last = rows_total - 1;
   const int hi = min(start + last / G, ctx - 1);
   int lo = 0;
-  if (a.window > 0) lo = max(0, start + item0 / G - a.window + 1);
+  lo = first_seen(a.window, start + item0 / G);
   int hi_w = -1, lo_w = 0;
   if (r0 < rows_total) {
     int last_w = r0 + 15;
     if (last_w >= rows_total) last_w = rows_total - 1;
     hi_w = min(start + last_w / G, ctx - 1);
-    if (a.window > 0) lo_w = max(0, start + r0 / G - a.window + 1);
+    lo_w = first_seen(a.window, start + r0 / G);
   }
 
   // the query row's elements 16 u + 4 g4 .. + 3, u = 0 .. DT - 1
@@ -180,7 +189,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
         for (int v = 0; v < 4; ++v) {
           const int j = t0 + 16 * st + 4 * g4 + v;
           bool vis = row_ok && j <= pos && j < ctx;
-          if (a.window > 0) vis = vis && (j > pos - a.window || j < keep);
+          if (a.window != 0) vis = vis && (j >= first_seen(a.window, pos) || j < keep);
           sc[v] = vis ? fmaf(slope, static_cast<float>(j - pos), capped(sc[v] * a.scale, a.cap)) : -INFINITY;
           tmax = fmaxf(tmax, sc[v]);
         }
@@ -333,7 +342,7 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
   const int token = seq_ok ? (cu_q ? cu_q[seq] : seq) : 0;
   const int pos = ctx - 1;
   int lo = 0;
-  if (a.window > 0 && pos - a.window + 1 > 0) lo = pos - a.window + 1;
+  if (pos >= 0) lo = first_seen(a.window, pos);
   // blocks of 64 keys from the block that holds `lo`; this cut takes blocks [b_lo, b_hi)
   // (counted in one unbroken range: the blocks of the kept keys, then those from `lo` on)
   const int keep = a.window > 0 ? a.keep : 0;

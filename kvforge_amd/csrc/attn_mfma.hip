@@ -84,6 +84,15 @@ struct MArgs {
   float cap;  // 0, or the scaled score s becomes cap * tanh(s / cap) (kernels with BIAS == 2)
 };
 
+// The first key a query at position `pos` sees: with a window w > 0 the key w - 1 before it, with
+// chunks (window < 0, chunks of -window positions counted from position 0) the first key of its
+// own chunk.  It does not fall as `pos` grows, so a range of rows sees from its first row's on.
+__device__ __forceinline__ int first_seen(int window, int pos) {
+  if (window > 0) return pos - window + 1 > 0 ? pos - window + 1 : 0;
+  if (window < 0) return pos - pos % (-window);
+  return 0;
+}
+
 // A walk over the blocks of 32 keys that a range of rows sees: blocks counted from `first` up to
 // `last` (in keys, multiples of 32; none if last < first) stand for the keys `at(count)`.
 struct Walk {
@@ -331,7 +340,7 @@ __device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int 
     rows.head[rt] = kvh * G + (rows.ok[rt] ? row - tok * G : 0);
     {  // the row's position is below the context length, so it is its last visible key
       const int pos = start + tok;
-      const int first = a.window > 0 && pos - a.window + 1 > 0 ? pos - a.window + 1 : 0;
+      const int first = first_seen(a.window, pos);
       rows.first[rt] = rows.ok[rt] ? first : -1;
       rows.span[rt] = rows.ok[rt] ? static_cast<unsigned>(pos - first) : 0u;
       rows.keep[rt] = rows.ok[rt] && a.window > 0 ? min(a.keep, pos + 1) : 0;
@@ -400,7 +409,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   int lo_w = 0, hi_w = -1;
   if (pos_max >= 0) {
     hi_w = pos_max < ctx - 1 ? pos_max : ctx - 1;
-    if (a.window > 0 && pos_min - a.window + 1 > 0) lo_w = pos_min - a.window + 1;
+    lo_w = first_seen(a.window, pos_min);
   }
   int lo_g = 0, hi_g = -1;
   if (seq_ok && wg_tile * 16 < qlen * G) {
@@ -408,7 +417,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
     if (t_hi > qlen - 1) t_hi = qlen - 1;
     hi_g = start + t_hi < ctx - 1 ? start + t_hi : ctx - 1;
     const int p_lo = start + wg_tile * 16 / G;
-    if (a.window > 0 && p_lo - a.window + 1 > 0) lo_g = p_lo - a.window + 1;
+    lo_g = first_seen(a.window, p_lo);
   }
   const float scale2 = a.scale * LOG2E;
   const int keep_w = a.window > 0 ? a.keep : 0;
@@ -502,7 +511,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
             kf[t][c] = as_frag(frag_lds[(buf * N_FRAG + t * DC + c) * KVF_WAVE + lane]);
 #pragma unroll
         for (int t = 0; t < DT; ++t) vf[t] = as_frag(frag_lds[(buf * N_FRAG + N_K + t) * KVF_WAVE + lane]);
-        const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
+        const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window != 0;
         block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
       }
     };
@@ -586,7 +595,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
         for (int c = 0; c < DC; ++c) kf[t][c] = as_frag(keep_first(kr[t][c], kl[t][c]));
 #pragma unroll
       for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(vr[t], vl));
-      const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
+      const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window != 0;
       block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
     }
   }
@@ -650,7 +659,7 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
   int lo = 0, hi = -1;
   if (pos_max >= 0) {
     hi = pos_max < ctx - 1 ? pos_max : ctx - 1;
-    if (a.window > 0 && pos_min - a.window + 1 > 0) lo = pos_min - a.window + 1;
+    lo = first_seen(a.window, pos_min);
   }
   // Blocks of 32 keys go round the waves of all cuts in turn: cut z, wave w take blocks
   // z * NW + w, then every (NW * splits)-th.  Without a window the first block is known before
@@ -700,12 +709,12 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
       for (int c = 0; c < DC; ++c) kf[t][c] = as_frag(keep_first(r.k[t][c], r.kl[t][c]));
 #pragma unroll
     for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(r.v[t], r.vl));
-    const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
+    const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window != 0;
     block_update<DT, 1, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
   };
   // Without a window the page lookups of the first blocks are asked for together with the
   // query and the context length, not after them: one round trip to memory less.
-  const bool early = a.window <= 0;
+  const bool early = a.window == 0;
   if (early) {
     locate(turn, pA);
     if (TWO) locate(turn + STEP, pB);

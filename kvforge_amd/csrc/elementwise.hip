@@ -1314,3 +1314,210 @@ KVF_EXPORT int kvf_rms_add_norm(int dtype, float* x, const float* y, const float
   if (dtype == 1) return rms_add_norm_launch<bf16_t>(x, y, w, eps, w2, eps2, out, m, h, s);
   return static_cast<int>(hipErrorInvalidValue);
 }
+
+// ----------------------------------------------------------------------------- whole-row q/k norm
+// Projected rows in fp32, `row_len` apart: H q heads of d elements, then KV k heads of d (then,
+// unless values are keys, KV v heads of d); of a head's d elements the first dk are real, the
+// rest padding.  Per token:
+//   q <- q + q_bias, k <- k + k_bias (fp32 vectors over the real elements, or null);
+//   the values are v's columns, or (v_from_k) the keys as they are here, before norm and rotation;
+//   q and k are each divided by the root mean square over *all* their real elements (every head
+//   at once, eps inside the root) and multiplied by weights qw [H dk], kw [KV dk];
+//   the first `rot` elements of every head are rotated in neighbouring pairs by the position's
+//   cos/sin row; q goes to q_out (rounded once), k and v to the token's place in the pages.
+// A workgroup takes a token.
+template <typename T>
+__global__ __launch_bounds__(256) void rownorm_rope_kvwrite_kernel(
+    const float* __restrict__ proj, const float* __restrict__ q_bias, const float* __restrict__ k_bias,
+    const float* __restrict__ qw, const float* __restrict__ kw, const int* __restrict__ positions,
+    const int* __restrict__ seq_of_token, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ block_table, T* __restrict__ q_out, int q_stride, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int dk, float eps, int v_from_k, RopeArgs a) {
+  __shared__ float scratch[2][16];
+  const int n = blockIdx.x;
+  const int p = positions[n];
+  const int half = a.rot / 2, d2 = a.d / 2;
+  const float* row = proj + static_cast<size_t>(n) * a.row_len;
+  const bool pos_ok = p >= 0 && p < a.table_len;
+  const float* cs = cos_t ? cos_t + static_cast<size_t>(pos_ok ? p : 0) * half : nullptr;
+  const float* sn = sin_t ? sin_t + static_cast<size_t>(pos_ok ? p : 0) * half : nullptr;
+  int page = -1, off = 0;
+  if (a.write_kv && pos_ok) {
+    const int seq = seq_of_token[n];
+    const int blk = p / a.block_size;
+    if (seq >= 0 && seq < a.n_seqs && blk < a.table_stride) {
+      page = block_table[static_cast<size_t>(seq) * a.table_stride + blk];
+      if (page >= a.num_blocks) page = -1;
+      off = p - blk * a.block_size;
+    }
+  }
+  float ssq = 0.f, ssk = 0.f;
+  for (int t = threadIdx.x; t < a.H * dk; t += blockDim.x) {
+    const int hh = t / dk, e = t - hh * dk;
+    const float x = row[hh * a.d + e] + (q_bias ? q_bias[t] : 0.f);
+    ssq = fmaf(x, x, ssq);
+  }
+  for (int t = threadIdx.x; t < a.KV * dk; t += blockDim.x) {
+    const int hh = t / dk, e = t - hh * dk;
+    const float x = row[(a.H + hh) * a.d + e] + (k_bias ? k_bias[t] : 0.f);
+    ssk = fmaf(x, x, ssk);
+  }
+  const float rq = 1.f / sqrtf(block_sum(ssq, scratch[0]) / static_cast<float>(a.H * dk) + eps);
+  const float rk = 1.f / sqrtf(block_sum(ssk, scratch[1]) / static_cast<float>(a.KV * dk) + eps);
+  for (int t = threadIdx.x; t < a.H * d2; t += blockDim.x) {
+    const int hh = t / d2, i = t - hh * d2, e = 2 * i;
+    const float* x = row + hh * a.d;
+    const int wi = hh * dk + e;
+    float y0 = e < dk ? (x[e] + (q_bias ? q_bias[wi] : 0.f)) * rq * qw[wi] : 0.f;
+    float y1 = e + 1 < dk ? (x[e + 1] + (q_bias ? q_bias[wi + 1] : 0.f)) * rq * qw[wi + 1] : 0.f;
+    if (e < a.rot && pos_ok && cs) {
+      const float c = cs[i], sv = sn[i];
+      const float t0 = y0 * c - y1 * sv, t1 = y1 * c + y0 * sv;
+      y0 = t0;
+      y1 = t1;
+    }
+    T* dst = q_out + static_cast<size_t>(n) * q_stride + hh * a.d + e;
+    Elem<T>::store(dst, y0);
+    Elem<T>::store(dst + 1, y1);
+  }
+  if (page < 0) return;
+  for (int t = threadIdx.x; t < a.KV * d2; t += blockDim.x) {
+    const int hh = t / d2, i = t - hh * d2, e = 2 * i;
+    const float* x = row + (a.H + hh) * a.d;
+    const int wi = hh * dk + e;
+    const float x0 = e < dk ? x[e] + (k_bias ? k_bias[wi] : 0.f) : 0.f;
+    const float x1 = e + 1 < dk ? x[e + 1] + (k_bias ? k_bias[wi + 1] : 0.f) : 0.f;
+    float y0 = e < dk ? x0 * rk * kw[wi] : 0.f;
+    float y1 = e + 1 < dk ? x1 * rk * kw[wi + 1] : 0.f;
+    if (e < a.rot && cs) {
+      const float c = cs[i], sv = sn[i];
+      const float t0 = y0 * c - y1 * sv, t1 = y1 * c + y0 * sv;
+      y0 = t0;
+      y1 = t1;
+    }
+    T* dst = k_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.block_size + off) * a.d + e;
+    Elem<T>::store(dst, y0);
+    Elem<T>::store(dst + 1, y1);
+    const float* vx = row + (a.H + a.KV + hh) * a.d;
+    const float v0 = v_from_k ? x0 : vx[e], v1 = v_from_k ? x1 : vx[e + 1];
+    T* vdst = v_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.d + e) * a.block_size + off;
+    Elem<T>::store(vdst, v0);
+    Elem<T>::store(vdst + a.block_size, v1);
+  }
+}
+#define ROWNORM_ARGS_DECL                                                                                    \
+  int dtype, const float *proj, const float *q_bias, const float *k_bias, const float *qw, const float *kw, \
+      const int *positions, const int *seq_of_token, const float *cos_t, const float *sin_t,                \
+      const int *block_table, void *q_out, int q_stride, void *k_pages, void *v_pages, int dk, float eps,   \
+      int v_from_k, int n, int H, int KV, int d, int rot, int table_len, int block_size, int table_stride,  \
+      int num_blocks, int write_kv, int n_seqs, int row_len, hipStream_t s
+// dtype of q_out and the pages: 0 = fp32, 1 = bf16
+KVF_EXPORT int kvf_rownorm_rope_kvwrite(ROWNORM_ARGS_DECL) {
+  if (n <= 0) return 0;
+  if (d % 2 || dk > d || dk <= 0 || rot > dk || rot % 2 || !qw || !kw || !q_out)
+    return static_cast<int>(hipErrorInvalidValue);
+  const RopeArgs a{ROPE_ARGS_PACK};
+  if (dtype == 0)
+    hipLaunchKernelGGL(rownorm_rope_kvwrite_kernel<float>, dim3(n), dim3(256), 0, s, proj, q_bias, k_bias, qw, kw,
+                       positions, seq_of_token, cos_t, sin_t, block_table, static_cast<float*>(q_out), q_stride,
+                       static_cast<float*>(k_pages), static_cast<float*>(v_pages), dk, eps, v_from_k, a);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(rownorm_rope_kvwrite_kernel<bf16_t>, dim3(n), dim3(256), 0, s, proj, q_bias, k_bias, qw, kw,
+                       positions, seq_of_token, cos_t, sin_t, block_table, static_cast<bf16_t*>(q_out), q_stride,
+                       static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages), dk, eps, v_from_k, a);
+  else
+    return static_cast<int>(hipErrorInvalidValue);
+  return kvf_last_error();
+}
+
+// ----------------------------------------------------------------------------- one gate per head
+// y[m, h * d + e] *= sigmoid(g[m, h]) * scale for h < H, e < d; g fp32, rows g_stride apart
+// (g null: y *= scale).
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ y, const float* __restrict__ g, int H, int d, int y_stride,
+                                 int g_stride, float scale, size_t total) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int cols = H * d;
+  const size_t m = idx / cols;
+  const int c = static_cast<int>(idx - m * cols);
+  T* yp = y + m * y_stride + c;
+  const float gate = g ? 1.f / (1.f + expf(-g[m * g_stride + c / d])) : 1.f;
+  Elem<T>::store(yp, Elem<T>::load(yp) * (gate * scale));
+}
+KVF_EXPORT int kvf_head_gate(int dtype, void* y, const float* g, int m, int H, int d, int y_stride, int g_stride,
+                             float scale, hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * H * d;
+  if (total == 0) return 0;
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256));
+  if (dtype == 0)
+    hipLaunchKernelGGL(head_gate_kernel<float>, grid, dim3(256), 0, s, static_cast<float*>(y), g, H, d, y_stride,
+                       g_stride, scale, total);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(head_gate_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<bf16_t*>(y), g, H, d, y_stride,
+                       g_stride, scale, total);
+  else
+    return static_cast<int>(hipErrorInvalidValue);
+  return kvf_last_error();
+}
+
+// ----------------------------------------------------------------------------- plain activations
+// out = act(x) element by element in fp32, rounded once.  act: 0 silu, 1 the tanh form of gelu,
+// 2 the square of relu.
+__device__ __forceinline__ float plain_act_f(int act, float z) {
+  if (act == 2) {
+    const float r = fmaxf(z, 0.f);
+    return r * r;
+  }
+  return act_f(act, z);
+}
+template <typename T>
+__global__ void plain_act_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total, int act) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < total) Elem<T>::store(out + i, plain_act_f(act, Elem<T>::load(x + i)));
+}
+KVF_EXPORT int kvf_plain_act(int dtype, const void* x, void* out, long total, int act, hipStream_t s) {
+  if (total <= 0) return 0;
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256));
+  if (dtype == 0)
+    hipLaunchKernelGGL(plain_act_kernel<float>, grid, dim3(256), 0, s, static_cast<const float*>(x),
+                       static_cast<float*>(out), static_cast<size_t>(total), act);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(plain_act_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<const bf16_t*>(x),
+                       static_cast<bf16_t*>(out), static_cast<size_t>(total), act);
+  else
+    return static_cast<int>(hipErrorInvalidValue);
+  return kvf_last_error();
+}
+
+// ----------------------------------------------------------------------------- gate per row
+// out[m, i] = act(gate_i) * up_i * sigmoid(rg[m]) with (gate, up) at (2i, 2i + 1) of the input
+// row; rg fp32, one number per row, rg_stride apart.  A feed-forward whose output is multiplied
+// by a number per token takes the number here, ahead of its (linear) down projection.
+template <typename T>
+__global__ void gated_act_rowgate_kernel(const T* __restrict__ gu, const float* __restrict__ rg, int rg_stride,
+                                         T* __restrict__ out, int inter, size_t total, int act) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t m = idx / inter;
+  const int i = static_cast<int>(idx - m * inter);
+  const T* row = gu + m * 2 * static_cast<size_t>(inter);
+  const float g = Elem<T>::load(row + 2 * i), u = Elem<T>::load(row + 2 * i + 1);
+  const float z = rg[m * rg_stride];
+  Elem<T>::store(out + idx, act_f(act, g) * u * (1.f / (1.f + expf(-z))));
+}
+KVF_EXPORT int kvf_gated_act_rowgate(int dtype, const void* gu, const float* rg, int rg_stride, void* out, int m,
+                                     int inter, int act, hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * inter;
+  if (total == 0) return 0;
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256));
+  if (dtype == 0)
+    hipLaunchKernelGGL(gated_act_rowgate_kernel<float>, grid, dim3(256), 0, s, static_cast<const float*>(gu), rg,
+                       rg_stride, static_cast<float*>(out), inter, total, act);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(gated_act_rowgate_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<const bf16_t*>(gu), rg,
+                       rg_stride, static_cast<bf16_t*>(out), inter, total, act);
+  else
+    return static_cast<int>(hipErrorInvalidValue);
+  return kvf_last_error();
+}

@@ -371,6 +371,19 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
     *reinterpret_cast<float4*>(xr + i + 4) = b;
   }
 }
+// A choice that a table makes: token id t uses the experts table[t, 0 .. top-1] (a row's entries
+// differ), each with weight 1 / top.  An id outside the table, or an entry that names no expert,
+// gives the pair (expert 0, weight 0): such a token adds nothing.
+__global__ void moe_table_kernel(const int* __restrict__ tokens, const int* __restrict__ table, int* __restrict__ sel,
+                                 float* __restrict__ wgt, int n, int vocab, int top, int E) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * top) return;
+  const int t = tokens[i / top];
+  const int e = t >= 0 && t < vocab ? table[static_cast<size_t>(t) * top + i % top] : -1;
+  const bool ok = e >= 0 && e < E;
+  sel[i] = ok ? e : 0;
+  wgt[i] = ok ? 1.f / static_cast<float>(top) : 0.f;
+}
 }  // namespace
 
 KVF_EXPORT int kvf_moe_topk(const float* z, int z_stride, const float* correction, int* sel, float* wgt,
@@ -379,6 +392,15 @@ KVF_EXPORT int kvf_moe_topk(const float* z, int z_stride, const float* correctio
   if (R <= 0 || R > MAX_PER_LANE * KVF_WAVE || top <= 0 || top > MAX_TOP || top > R)
     return static_cast<int>(hipErrorInvalidValue);
   hipLaunchKernelGGL(moe_topk_kernel, dim3(n), dim3(KVF_WAVE), 0, s, z, z_stride, correction, sel, wgt, R, top);
+  return kvf_last_error();
+}
+
+KVF_EXPORT int kvf_moe_table(const int* tokens, const int* table, int* sel, float* wgt, int n, int vocab, int top,
+                             int E, hipStream_t s) {
+  if (n <= 0) return 0;
+  if (vocab <= 0 || top <= 0 || top > MAX_TOP || E <= 0) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(moe_table_kernel, dim3((n * top + 255) / 256), dim3(256), 0, s, tokens, table, sel, wgt, n,
+                     vocab, top, E);
   return kvf_last_error();
 }
 

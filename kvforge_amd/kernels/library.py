@@ -48,6 +48,7 @@ MODULES: dict[str, list[str]] = {
     "moe": ["moe.hip"],
     "latent": ["latent.hip"],
     "wkv": ["wkv.hip"],
+    "linmem": ["linmem.hip"],
 }
 
 

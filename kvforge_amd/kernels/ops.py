@@ -495,6 +495,110 @@ def qknorm_rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token
           1 if write_kv else 0, n_seqs, qkv.shape[1], _stream()), "qknorm_rope_kvwrite")
 
 
+def rownorm_rope_kvwrite(proj: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
+                         seq_of_token: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
+                         block_table: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                         num_heads: int, num_kv_heads: int, head_dim: int, q_weight: torch.Tensor,
+                         k_weight: torch.Tensor, norm_dim: int, eps: float,
+                         q_bias: torch.Tensor | None = None, k_bias: torch.Tensor | None = None,
+                         values_are_keys: bool = False, write_kv: bool = True) -> None:
+    """From projected rows in fp32 (``proj [n, >= (H + KV) d]``, or ``(H + 2 KV) d`` with values
+    of their own): biases on q and k (fp32 over the heads' first ``norm_dim`` elements, or
+    ``None``); q and k each divided by the root mean square over *all* their elements at once
+    (every head, ``eps`` inside the root) and multiplied by ``q_weight [H * norm_dim]`` /
+    ``k_weight [KV * norm_dim]``; the rotation of neighbouring pairs; q to ``q_out [n, H * d]``,
+    k and the values to the pages.  ``values_are_keys``: a token's values are its keys as they
+    stand after the bias, before norm and rotation."""
+    n = proj.shape[0]
+    H, KV, d = int(num_heads), int(num_kv_heads), int(head_dim)
+    _check(proj, "proj", F32, (n, None))
+    need = (H + (KV if values_are_keys else 2 * KV)) * d
+    if proj.shape[1] < need:
+        raise KernelError(f"rownorm_rope_kvwrite: rows of {proj.shape[1]} elements do not hold {need}")
+    if not 0 < norm_dim <= d <= 256 or d % 2:
+        raise KernelError(f"rownorm_rope_kvwrite: heads of {norm_dim} in {d} elements (even, at most 256)")
+    _check(q_out, "q_out", None, (n, H * d), contiguous=False)
+    if q_out.stride(1) != 1:
+        raise KernelError("rownorm_rope_kvwrite: rows of q_out must be dense")
+    _check(positions, "positions", I32, (None,))
+    _check(seq_of_token, "seq_of_token", I32, (None,))
+    if positions.shape[0] < n or seq_of_token.shape[0] < n:
+        raise KernelError("rownorm_rope_kvwrite: positions / seq_of_token shorter than the batch")
+    cos_p, sin_p, rot, table_len = _rotary_tables(cos, sin, d, "rownorm_rope_kvwrite")
+    if rot > norm_dim:
+        raise KernelError(f"rownorm_rope_kvwrite: rotary width {rot} beyond the head's {norm_dim} elements")
+    _check(q_weight, "q_weight", F32, (H * norm_dim,))
+    _check(k_weight, "k_weight", F32, (KV * norm_dim,))
+    if q_bias is not None:
+        _check(q_bias, "q_bias", F32, (H * norm_dim,))
+    if k_bias is not None:
+        _check(k_bias, "k_bias", F32, (KV * norm_dim,))
+    _check(block_table, "block_table", I32, (None, None))
+    n_seqs, stride = block_table.shape
+    _check(k_pages, "k_pages", q_out.dtype, (None, KV, None, d))
+    nb, _, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", q_out.dtype, (nb, KV, d, bs))
+    f = _fn("elementwise", "kvf_rownorm_rope_kvwrite",
+            [c_int] + [c_void_p] * 11 + [c_int, c_void_p, c_void_p, c_int, c_float] + [c_int] * 13 + [c_void_p])
+    _ok(f(_tcode(q_out.dtype), proj.data_ptr(), q_bias.data_ptr() if q_bias is not None else None,
+          k_bias.data_ptr() if k_bias is not None else None, q_weight.data_ptr(), k_weight.data_ptr(),
+          positions.data_ptr(), seq_of_token.data_ptr(), cos_p, sin_p, block_table.data_ptr(), q_out.data_ptr(),
+          q_out.stride(0) if n > 1 else H * d, k_pages.data_ptr(), v_pages.data_ptr(), int(norm_dim), float(eps),
+          1 if values_are_keys else 0, n, H, KV, d, rot, table_len, bs, stride, nb, 1 if write_kv else 0, n_seqs,
+          proj.shape[1], _stream()), "rownorm_rope_kvwrite")
+
+
+def head_gate(y: torch.Tensor, gate: torch.Tensor | None, heads: int, head_dim: int, scale: float = 1.0) -> None:
+    """``y[m, h * d + e] *= sigmoid(gate[m, h]) * scale``: one gate number per head.  ``y [M, H * d]``
+    with dense rows; ``gate`` fp32 ``[M, >= H]`` with dense rows (a block of columns of a wider
+    product is fine), or ``None`` for the scale alone."""
+    m = y.shape[0]
+    H, d = int(heads), int(head_dim)
+    _check(y, "y", None, (m, H * d), contiguous=False)
+    if y.stride(1) != 1:
+        raise KernelError("head_gate: rows of y must be dense")
+    if gate is None:
+        f = _fn("elementwise", "kvf_head_gate", [c_int, c_void_p, c_void_p] + [c_int] * 5 + [c_float, c_void_p])
+        _ok(f(_tcode(y.dtype), y.data_ptr(), None, m, H, d, y.stride(0) if m > 1 else H * d, 0, float(scale),
+              _stream()), "head_gate")
+        return
+    _check(gate, "gate", F32, (m, None), contiguous=False)
+    if gate.shape[1] < H or gate.stride(1) != 1:
+        raise KernelError("head_gate: a gate per head in dense rows")
+    f = _fn("elementwise", "kvf_head_gate", [c_int, c_void_p, c_void_p] + [c_int] * 5 + [c_float, c_void_p])
+    _ok(f(_tcode(y.dtype), y.data_ptr(), gate.data_ptr(), m, H, d, y.stride(0) if m > 1 else H * d,
+          gate.stride(0) if m > 1 else gate.shape[1], float(scale), _stream()), "head_gate")
+
+
+PLAIN_ACTIVATIONS = dict(ACTIVATIONS, relu2=2)
+
+
+def plain_act(x: torch.Tensor, out: torch.Tensor, activation: str) -> None:
+    """``out = act(x)`` element by element in fp32, rounded once (``out`` may be ``x``).
+    ``activation``: ``"silu"``, ``"gelu_tanh"`` or ``"relu2"`` (the square of relu)."""
+    if activation not in PLAIN_ACTIVATIONS:
+        raise KernelError(f"plain_act: unknown activation {activation!r}; known: {sorted(PLAIN_ACTIVATIONS)}")
+    _check(x, "x")
+    _check(out, "out", x.dtype, tuple(x.shape))
+    f = _fn("elementwise", "kvf_plain_act", [c_int, c_void_p, c_void_p, c_long, c_int, c_void_p])
+    _ok(f(_tcode(x.dtype), x.data_ptr(), out.data_ptr(), x.numel(), PLAIN_ACTIVATIONS[activation], _stream()),
+        "plain_act")
+
+
+def gated_act_rowgate(gate_up: torch.Tensor, row_gate: torch.Tensor, out: torch.Tensor, activation: str) -> None:
+    """``out[m, i] = act(gate_i) * up_i * sigmoid(row_gate[m])`` with (gate, up) at ``(2i, 2i + 1)``
+    of the input row; ``row_gate`` fp32 ``[M, >= 1]`` (its first column counts)."""
+    m, two_i = gate_up.shape
+    if two_i % 2 or activation not in ACTIVATIONS:
+        raise KernelError(f"gated_act_rowgate: an even width and one of {sorted(ACTIVATIONS)}")
+    _check(gate_up, "gate_up", None, (m, two_i))
+    _check(out, "out", gate_up.dtype, (m, two_i // 2))
+    _check(row_gate, "row_gate", F32, (m, None), contiguous=False)
+    f = _fn("elementwise", "kvf_gated_act_rowgate", [c_int, c_void_p, c_void_p, c_int, c_void_p] + [c_int] * 3 + [c_void_p])
+    _ok(f(_tcode(out.dtype), gate_up.data_ptr(), row_gate.data_ptr(), row_gate.stride(0) if m > 1 else 1,
+          out.data_ptr(), m, two_i // 2, ACTIVATIONS[activation], _stream()), "gated_act_rowgate")
+
+
 # ------------------------------------------------------------------------------ matrix products
 # Rows of the left operand up to which the weight-streaming MFMA kernel is used for bf16.  Over
 # tiled weights it measured faster than the library's product up to 32 rows on the shapes of a
@@ -1005,6 +1109,15 @@ def _keep_first(window: int, keep_first: int) -> int:
     return keep if int(window) > 0 else 0
 
 
+def _mask_arg(window: int, chunk: int) -> int:
+    """What the attention kernels take as their mask: a window ``w`` as ``w``, chunks of ``c``
+    positions as ``-c``, neither as 0."""
+    window, chunk = int(window or 0), int(chunk or 0)
+    if window < 0 or chunk < 0 or (window and chunk):
+        raise KernelError(f"attention: a window ({window}) or chunks ({chunk}), not negative and not both")
+    return -chunk if chunk else window
+
+
 def _gate_args(gate, q: torch.Tensor, cols: int):
     """(pointer, row stride) of an output gate, or (None, 0)."""
     if gate is None:
@@ -1052,7 +1165,8 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  head_dim: int, scale: float, window: int = 0,
                  slopes: torch.Tensor | None = None, rows_per_item: int | None = None,
                  keep_first: int = 0, gate: torch.Tensor | None = None,
-                 sinks: torch.Tensor | None = None, score_cap: float | None = None) -> None:
+                 sinks: torch.Tensor | None = None, score_cap: float | None = None,
+                 chunk: int = 0) -> None:
     """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 3]`` rows
     (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
     an item covers ``rows_per_item`` of them (what ``prefill_rows_per_item`` gave when the rows
@@ -1067,8 +1181,11 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     ``sinks``: fp32 ``[H]``; the softmax's denominator of head ``h`` then holds one more term
     ``exp(sinks[h])``, a key without a value whose score is not scaled.
     ``score_cap``: the scaled score ``s`` becomes ``score_cap * tanh(s / score_cap)`` (the
-    matrix-core kernels have it without sinks and slopes only)."""
+    matrix-core kernels have it without sinks and slopes only).
+    ``chunk``: positions are cut into chunks of so many, counted from position 0 of the sequence,
+    and a query sees only the keys of its own chunk (instead of a window, not beside one)."""
     H, KV, d = num_heads, num_kv_heads, head_dim
+    window = _mask_arg(window, chunk)
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     cap = _score_cap(score_cap, sinks, slopes, attention_on_matrix_cores(q.dtype, k_pages.shape[2]))
     _check(work, "work", I32, (None, 3))
@@ -1111,7 +1228,8 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
                 token_is_seq: bool = False, slopes: torch.Tensor | None = None,
                 keep_first: int = 0, gate: torch.Tensor | None = None,
-                sinks: torch.Tensor | None = None, score_cap: float | None = None) -> None:
+                sinks: torch.Tensor | None = None, score_cap: float | None = None,
+                chunk: int = 0) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
     each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  The key
     range may be cut into ``splits`` runs; ``workspace`` then holds fp32 partial accumulators
@@ -1120,8 +1238,10 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     single tokens), which spares the matrix-core kernel a dependent load.  ``slopes``: as in
     ``attn_prefill``; ``keep_first`` and ``gate`` likewise (the matrix-core kernels only: the
     32-bit path is given no gate, its caller gates the rows afterwards); ``sinks`` likewise (all
-    kernels; with cuts the term joins the sum where the cuts are merged); ``score_cap`` likewise."""
+    kernels; with cuts the term joins the sum where the cuts are merged); ``score_cap`` and
+    ``chunk`` likewise."""
     H, KV, d = num_heads, num_kv_heads, head_dim
+    window = _mask_arg(window, chunk)
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     cap = _score_cap(score_cap, sinks, slopes, attention_on_matrix_cores(q.dtype, k_pages.shape[2]))
     sl = _slopes_ptr(slopes, H, q)
@@ -1592,6 +1712,154 @@ def moe_grouped(x: torch.Tensor, w_gate_up: "StreamedWeight", w_down: "StreamedW
           scratch["where"].data_ptr(), scratch["order"].data_ptr(), scratch["tiles"].data_ptr(),
           scratch["num_tiles"].data_ptr(), max_tiles, scratch["act"].data_ptr(), scratch["y"].data_ptr(),
           residual.data_ptr(), _stream()), "moe_grouped")
+
+
+
+def moe_table(tokens: torch.Tensor, table: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+              experts: int) -> None:
+    """A choice made by a table: token id ``t`` uses the experts ``table[t]`` (int32
+    ``[vocab, top]``), each with weight ``1 / top``; ``chosen [N, top]`` (int32) and
+    ``weights [N, top]`` (fp32) as ``moe_topk`` leaves them."""
+    n, top = chosen.shape
+    _check(tokens, "tokens", I32, (None,))
+    if tokens.shape[0] < n:
+        raise KernelError("moe_table: fewer token ids than rows")
+    _check(table, "table", I32, (None, top))
+    _check(chosen, "chosen", I32, (n, top))
+    _check(weights, "weights", F32, (n, top))
+    if not 0 < top <= MOE_MAX_TOP:
+        raise KernelError(f"moe_table: up to {MOE_MAX_TOP} choices, got {top}")
+    f = _fn("moe", "kvf_moe_table", [c_void_p] * 4 + [c_int] * 4 + [c_void_p])
+    _ok(f(tokens.data_ptr(), table.data_ptr(), chosen.data_ptr(), weights.data_ptr(), n, table.shape[0], top,
+          int(experts), _stream()), "moe_table")
+
+
+# ------------------------------------------------------------------------------ linear-attention memory
+# Runs of at least LINMEM_MULTI_FROM tokens are cut into chunks of LINMEM_CHUNK tokens that go side
+# by side (three passes); shorter runs go token by token in one workgroup per head and slice.
+LINMEM_CHUNK = 16
+LINMEM_MULTI_FROM = 64
+
+
+def linmem_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
+    """fp32 numbers of a request's slot: every head's ``S [key_dim, value_dim]``."""
+    return int(heads) * int(key_dim) * int(value_dim)
+
+
+def linmem_multi_plan(q_lens, multi_from: int = LINMEM_MULTI_FROM) -> tuple[list[int], list[int]]:
+    """For the runs of at least ``multi_from`` tokens among ``q_lens`` (a step's runs in sequence
+    order): the flat rows ``(sequence, first token, tokens, 0)`` of their chunks and
+    ``(sequence, first chunk, chunks)`` of the runs, as ``linmem_scan(multi=...)`` wants them."""
+    chunks: list[int] = []
+    runs: list[int] = []
+    start = 0
+    for seq, q in enumerate(q_lens):
+        if q >= multi_from:
+            first = len(chunks) // 4
+            for t in range(0, q, LINMEM_CHUNK):
+                chunks += [seq, start + t, min(LINMEM_CHUNK, q - t), 0]
+            runs += [seq, first, len(chunks) // 4 - first]
+        start += q
+    return chunks, runs
+
+
+def linmem_multi_scratch(n_chunks: int, heads: int, key_dim: int, value_dim: int) -> dict[str, tuple]:
+    """(shape, dtype) of the scratch tensors the passes over all chunks need, by name."""
+    return {"G": ((n_chunks, int(heads), int(key_dim), int(value_dim)), F32),
+            "D": ((n_chunks, int(heads), int(key_dim)), F32)}
+
+
+def linmem_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor,
+                cu_q: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor,
+                out: torch.Tensor, n_seqs: int, heads: int, key_dim: int, value_dim: int,
+                gate_bias: torch.Tensor | None = None, tau: float | None = None, q_scale: float = 1.0,
+                k_scale: float = 1.0, multi: dict | None = None, short_runs: bool = True,
+                cos: torch.Tensor | None = None, sin: torch.Tensor | None = None) -> None:
+    """The recurrence ``S_ij <- a_i S_ij + k_i v_j``, ``o_j = sum_i q_i S_ij`` (the output sees
+    its own token) over every query run, in fp32, from and to the sequences' state slots (a run
+    at position 0 starts from zeros whatever its slot holds; a sequence without a slot starts
+    from zeros and keeps nothing).  ``q, k [n, heads * key_dim]`` and ``v [n, heads * value_dim]``
+    are dense rows (views of wider rows are fine).  With ``cos`` / ``sin`` (fp32 tables by
+    position) the first elements of every q and k head are rotated in neighbouring pairs first, in
+    fp32; then q and k are multiplied by ``q_scale`` / ``k_scale`` in fp32.  The decays: with ``tau`` given, ``decay`` is fp32 ``[n, >= heads *
+    key_dim]`` pre-activations and ``a = sigmoid(decay + gate_bias)^(1/tau)``; otherwise
+    ``decay`` is fp32 ``[heads * key_dim]``, constants.  ``out`` fp32 ``[n, heads * value_dim]``.
+    ``multi``: ``chunks`` and ``runs`` (int32 device tensors of ``linmem_multi_plan``'s rows) and
+    the scratch ``G``, ``D``: those runs go chunk by chunk side by side and the token-by-token
+    kernel leaves them alone; it is not launched at all with ``short_runs=False``."""
+    n = q.shape[0]
+    H, dk, dv = int(heads), int(key_dim), int(value_dim)
+    for t, name, w in ((q, "q", H * dk), (k, "k", H * dk), (v, "v", H * dv)):
+        _check(t, name, q.dtype, (n, w), contiguous=False)
+        if t.stride(1) != 1:
+            raise KernelError(f"linmem_scan: rows of {name} must be dense")
+    gated = tau is not None
+    if gated:
+        _check(decay, "decay", F32, (n, None), contiguous=False)
+        if decay.shape[1] < H * dk or decay.stride(1) != 1 or not tau > 0:
+            raise KernelError("linmem_scan: gate rows too short, not dense, or tau not positive")
+        if gate_bias is not None:
+            _check(gate_bias, "gate_bias", F32, (H * dk,))
+    else:
+        _check(decay, "decay", F32, (H * dk,))
+        if gate_bias is not None:
+            raise KernelError("linmem_scan: a gate bias goes with gates (tau)")
+    _check(out, "out", F32, (n, H * dv))
+    _check(state, "state", F32, (None, None))
+    if state.shape[1] < H * dk * dv or not 0 < dk <= 256 or dv <= 0:
+        raise KernelError(f"linmem_scan: heads of {dk} x {dv} (key size at most 256) need slots of {H * dk * dv} floats")
+    for t, name in ((cu_q, "cu_q"), (positions, "positions"), (slot_ids, "slot_ids")):
+        _check(t, name, I32, (None,))
+    if cu_q.shape[0] < n_seqs + 1 or slot_ids.shape[0] < n_seqs or positions.shape[0] < n:
+        raise KernelError("linmem_scan: batch arrays shorter than the batch")
+    stride = lambda t, w: t.stride(0) if n > 1 else w  # noqa: E731
+    cos_p, sin_p, rot, table_len = _rotary_tables(cos, sin, dk, "linmem_scan")
+    common = (_tcode(q.dtype), q.data_ptr(), k.data_ptr(), v.data_ptr(), decay.data_ptr(),
+              gate_bias.data_ptr() if gate_bias is not None else None, cos_p, sin_p, rot, table_len,
+              cu_q.data_ptr(), positions.data_ptr(),
+              slot_ids.data_ptr(), state.data_ptr(), out.data_ptr(), int(n_seqs), H, dk, dv, state.shape[0],
+              state.shape[1], stride(q, H * dk), stride(k, H * dk), stride(v, H * dv), 1 if gated else 0,
+              (decay.stride(0) if n > 1 else decay.shape[1]) if gated else 0,
+              1.0 / float(tau) if gated else 1.0, float(q_scale), float(k_scale))
+    types = [c_int] + [c_void_p] * 7 + [c_int] * 2 + [c_void_p] * 5 + [c_int] * 11 + [c_float] * 3
+    if short_runs or multi is None:
+        f = _fn("linmem", "kvf_linmem_scan", types + [c_int, c_void_p])
+        _ok(f(*common, LINMEM_MULTI_FROM if multi is not None else 0, _stream()), "linmem_scan")
+    if multi is None:
+        return
+    chunks, runs, G, D = multi["chunks"], multi["runs"], multi["G"], multi["D"]
+    _check(chunks, "chunks", I32, (None, 4))
+    _check(runs, "runs", I32, (None, 3))
+    nc = chunks.shape[0]
+    _check(G, "G", F32, (None, H, dk, dv))
+    _check(D, "D", F32, (None, H, dk))
+    if G.shape[0] < nc or D.shape[0] < nc:
+        raise KernelError("linmem_scan: scratch for fewer chunks than the plan has")
+    f = _fn("linmem", "kvf_linmem_chunks", types + [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p])
+    _ok(f(*common, chunks.data_ptr(), nc, runs.data_ptr(), runs.shape[0], G.data_ptr(), D.data_ptr(), _stream()),
+        "linmem_chunks")
+
+
+def linmem_out(heads_raw: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor | None, eps: float,
+               out: torch.Tensor, heads: int, value_dim: int, scale: float = 1.0) -> None:
+    """``out[n, h, :] = o / rms(o) * weight * silu(gate[n, h, :]) * scale`` for the raw heads
+    ``o = heads_raw[n, h, :]`` (fp32), the root mean square per head with ``eps`` inside the
+    root; ``weight`` fp32 ``[value_dim]`` shared by the heads, or ``None`` for none.  ``gate``:
+    dense rows of ``out``'s type (a view of wider rows is fine)."""
+    n = heads_raw.shape[0]
+    H, dv = int(heads), int(value_dim)
+    _check(heads_raw, "heads_raw", F32, (n, H * dv))
+    if weight is not None:
+        _check(weight, "weight", F32, (dv,))
+    _check(out, "out", None, (n, H * dv))
+    _check(gate, "gate", out.dtype, (n, H * dv), contiguous=False)
+    if gate.stride(1) != 1:
+        raise KernelError("linmem_out: gate rows must be dense")
+    f = _fn("linmem", "kvf_linmem_out", [c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_float, c_void_p]
+            + [c_int] * 3 + [c_void_p])
+    _ok(f(_tcode(out.dtype), heads_raw.data_ptr(), gate.data_ptr(), gate.stride(0) if n > 1 else H * dv,
+          weight.data_ptr() if weight is not None else None, float(eps), float(scale), out.data_ptr(), n, H, dv,
+          _stream()), "linmem_out")
 
 
 # ------------------------------------------------------------------------------ sampling

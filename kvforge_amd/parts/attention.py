@@ -102,7 +102,24 @@ class PagedAttention(Mixer):
     mask and softmax.
     ``q_temp``: ``(coef, every)``; the query of position ``p`` is multiplied by
     ``1 + coef * ln(floor((p + 1) / every) + 1)``, in the kernel that norms q and k (so it goes
-    with ``qk_norm``)."""
+    with ``qk_norm``).
+    ``row_norm``: ``(name of q's weight, name of k's weight, eps)`` under the prefix: q as a whole
+    (all heads at once) and k as a whole are each divided by their root mean square and
+    multiplied by a weight vector of their full size (``[heads * head_dim]``,
+    ``[kv heads * head_dim]``), before the rotation; the projection's sums are kept in fp32 up to
+    there.  ``bias``: ``(name of q's bias, name of k's bias)`` under the prefix, added to the
+    projections in fp32 (goes with ``row_norm``, whose kernel adds them).
+    ``values_are_keys``: there is no value projection; a token's values are its keys as they
+    leave the projection (bias included), before norm and rotation (goes with ``row_norm`` and a
+    rotation of neighbouring pairs or none).
+    ``chunk``: instead of a window, positions are cut into chunks of so many, counted from
+    position 0 of the sequence, and a query sees only the keys of its own chunk; pages wholly
+    behind the chunk are given back.
+    ``head_gate``: name of a matrix ``[num_heads, hidden]`` under the prefix: head ``h``'s output is
+    multiplied by ``sigmoid(W x)_h``, one number per head, from the same input as the
+    projections; a product of its own with fp32 sums stored in fp32.
+    ``out_scale``: a constant on the heads' outputs, applied in fp32 ahead of the (linear) output
+    projection."""
 
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "g": "g_proj.weight"}
@@ -116,7 +133,10 @@ class PagedAttention(Mixer):
                  value_dim: int | None = None, gated: bool = False, own_kv: bool = True,
                  names: dict[str, str] | None = None,
                  qk_norm: tuple[str, str, float] | None = None, sink: str | None = None,
-                 score_cap: float | None = None, q_temp: tuple[float, int] | None = None) -> None:
+                 score_cap: float | None = None, q_temp: tuple[float, int] | None = None,
+                 row_norm: tuple[str, str, float] | None = None, bias: tuple[str, str] | None = None,
+                 values_are_keys: bool = False, chunk: int | None = None, head_gate: str | None = None,
+                 out_scale: float = 1.0) -> None:
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.dk = int(head_dim)
@@ -133,6 +153,9 @@ class PagedAttention(Mixer):
         self.rotary = rotary
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.dk)
         self.window = int(window) if window else None
+        self.chunk = int(chunk) if chunk else None
+        if self.chunk is not None and (self.chunk < 0 or self.window is not None):
+            raise ValueError("chunks are positive and take the place of a window")
         self.keep_first = int(keep_first) if self.window else 0
         if self.keep_first < 0:
             raise ValueError(f"keep_first must not be negative, got {keep_first}")
@@ -152,12 +175,25 @@ class PagedAttention(Mixer):
         self.q_temp = (float(q_temp[0]), int(q_temp[1])) if q_temp else None
         if self.q_temp is not None and (qk_norm is None or self.q_temp[1] < 1):
             raise ValueError("q_temp goes with qk_norm and a positive step")
-        self.cache_spec = CacheSpec(attention_pages(self.KV, self.d), self.window, self.keep_first)
+        self.row_norm, self.bias, self.values_are_keys = row_norm, bias, bool(values_are_keys)
+        if row_norm is not None and (qk_norm is not None or not own_kv or gated):
+            raise ValueError("a norm over whole q and k rows goes with key projections of the mixer's own, "
+                             "without a norm per head and without an element-wise gate")
+        if (bias is not None or self.values_are_keys) and row_norm is None:
+            raise ValueError("biases on q and k, and values that are the keys, go with row_norm")
+        if self.values_are_keys and (self.dv != self.dk or (rotary is not None and not rotary.interleaved)):
+            raise ValueError("values that are the keys have the keys' size and order (a rotation of "
+                             "neighbouring pairs, or none)")
+        self.head_gate, self.out_scale = head_gate, float(out_scale)
+        self.q_bias = self.k_bias = self.w_head_gate = None
+        # a chunk's keys all lie within the last `chunk` positions
+        self.cache_spec = CacheSpec(attention_pages(self.KV, self.d), self.window or self.chunk, self.keep_first)
         self.w_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
 
     def _matrices(self) -> list[str]:
-        return ["q"] + (["k", "v"] if self.own_kv else []) + (["g"] if self.gated else [])
+        kv = (["k"] if self.values_are_keys else ["k", "v"]) if self.own_kv else []
+        return ["q"] + kv + (["g"] if self.gated else [])
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         h, H, KV = self.hidden, self.H, self.KV
@@ -170,6 +206,14 @@ class PagedAttention(Mixer):
             out[self._name(self.qk_norm[1])] = WeightSpec((self.dk,), init="norm", std=0.1)
         if self.sink is not None:
             out[self._name(self.sink)] = WeightSpec((H,), std=1.0)
+        if self.row_norm is not None:
+            out[self._name(self.row_norm[0])] = WeightSpec((H * self.dk,), init="norm", std=0.1)
+            out[self._name(self.row_norm[1])] = WeightSpec((KV * self.dk,), init="norm", std=0.1)
+        if self.bias is not None:
+            out[self._name(self.bias[0])] = WeightSpec((H * self.dk,), std=0.5)
+            out[self._name(self.bias[1])] = WeightSpec((KV * self.dk,), std=0.5)
+        if self.head_gate is not None:
+            out[self._name(self.head_gate)] = WeightSpec((H, h))
         return out
 
     def _padded_heads(self, w: torch.Tensor, heads: int, size: int, perm=None) -> torch.Tensor:
@@ -193,8 +237,9 @@ class PagedAttention(Mixer):
         perm = self.pair_permutation()
         rows = [self._padded_heads(mats["q"], self.H, self.dk, perm)]
         if self.own_kv:
-            rows += [self._padded_heads(mats["k"], self.KV, self.dk, perm),
-                     self._padded_heads(mats["v"], self.KV, self.dv)]
+            rows.append(self._padded_heads(mats["k"], self.KV, self.dk, perm))
+            if not self.values_are_keys:
+                rows.append(self._padded_heads(mats["v"], self.KV, self.dv))
         if self.gated:
             rows.append(self._padded_heads(mats["g"], self.H, self.dv))
         # one product for all projections: rows of q heads, then k heads, then v heads, then
@@ -212,6 +257,18 @@ class PagedAttention(Mixer):
             self.k_norm_w = tensors[self._name(self.qk_norm[1])].float().contiguous()
         if self.sink is not None:
             self.sinks = tensors[self._name(self.sink)].float().contiguous()
+        if self.row_norm is not None:
+            # weights and biases go by (head, element): in the order the rows of q and k were given
+            def by_head(name: str, heads: int) -> torch.Tensor:
+                return tensors[self._name(name)].float().view(heads, self.dk)[:, perm.to(w_o.device)].reshape(-1).contiguous()
+            self.q_norm_w, self.k_norm_w = by_head(self.row_norm[0], self.H), by_head(self.row_norm[1], self.KV)
+            if self.bias is not None:
+                self.q_bias, self.k_bias = by_head(self.bias[0], self.H), by_head(self.bias[1], self.KV)
+        if self.head_gate is not None:
+            # one row per head, padded with zero rows to a multiple of 16 (which every product
+            # kernel takes); in the engine's type, its 32-bit sums are stored in fp32
+            g = tensors[self._name(self.head_gate)]
+            self.w_head_gate = torch.cat([g, g.new_zeros(-(-self.H // 16) * 16 - self.H, self.hidden)], dim=0).contiguous()
         if self.score_slopes is not None:
             self.slopes = torch.tensor(self.score_slopes, dtype=torch.float32, device=self.w_o.device)
 
@@ -241,10 +298,10 @@ class PagedAttention(Mixer):
     def _plain(self) -> bool:
         """Whether the product holds q, k and v and nothing else, and nothing but the rotation
         lies between it and the cache."""
-        return self.own_kv and not self.gated and self.qk_norm is None
+        return self.own_kv and not self.gated and self.qk_norm is None and self.row_norm is None
 
     def absorb_norm(self, norm) -> bool:
-        if self._hooked() or not self._plain():
+        if self._hooked() or not self._plain() or self.head_gate is not None:
             return False
         if self.norm_eps is not None or not getattr(norm, "foldable_into", lambda m: False)(self.w_qkv):
             return False
@@ -263,13 +320,19 @@ class PagedAttention(Mixer):
                    for t in (*map(ops.plain_of, (self.w_qkv, self.w_o)), *self._small()) if t is not None)
 
     def _small(self) -> list[torch.Tensor]:
-        return [t for t in (self.q_norm_w, self.k_norm_w, self.sinks) if t is not None]
+        gate = ops.plain_of(self.w_head_gate) if self.w_head_gate is not None else None
+        return [t for t in (self.q_norm_w, self.k_norm_w, self.sinks, self.q_bias, self.k_bias, gate)
+                if t is not None]
 
     def held_tensors(self) -> list[torch.Tensor]:
-        return ops.copies_of(self.w_qkv) + ops.copies_of(self.w_o) + self._small()
+        gate = ops.copies_of(self.w_head_gate) if self.w_head_gate is not None else []
+        return (ops.copies_of(self.w_qkv) + ops.copies_of(self.w_o) + gate
+                + [t for t in self._small() if t.dim() == 1])
 
     def seal(self) -> None:
         self.w_qkv, self.w_o = ops.streamed(ops.plain_of(self.w_qkv)), ops.streamed(ops.plain_of(self.w_o))
+        if self.w_head_gate is not None:
+            self.w_head_gate = ops.streamed(ops.plain_of(self.w_head_gate))
 
     # ------------------------------------------------------------------ launch planning
     def launch_key(self, shape) -> tuple[int, int]:
@@ -277,7 +340,8 @@ class PagedAttention(Mixer):
         on besides the padded batch size.  A cell is ``KEYS_PER_CUT`` keys of the longest
         context (of the window, for a windowed layer), and the plan is made for the cell's lower
         edge."""
-        ctx = min(shape.max_ctx, self.window + self.keep_first) if self.window else shape.max_ctx
+        seen = self.window or self.chunk
+        ctx = min(shape.max_ctx, seen + self.keep_first) if seen else shape.max_ctx
         cell = min(ctx // KEYS_PER_CUT, MAX_CUTS)
         return cell, skew_cuts(max(cell * KEYS_PER_CUT, 1), shape.sum_ctx, shape.n)
 
@@ -341,7 +405,7 @@ class PagedAttention(Mixer):
             normed = ws.buf("normed", (n, self.hidden), act)
             ops.rmsnorm(x, None, rms, normed, add=step.take_owed(residual))
             x, rms = normed, None
-        fused = (not self._hooked() and self.qk_norm is None
+        fused = (not self._hooked() and self.qk_norm is None and self.row_norm is None
                  and ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True)
                  and layer.k_pages.dtype == torch.bfloat16)
         if fused and rms is not None:
@@ -362,6 +426,17 @@ class PagedAttention(Mixer):
                               layer.k_pages, layer.v_pages, H, KV if self.own_kv else 0, d,
                               write_kv=layer.owns_cache and self.own_kv, rms_eps=rms, a_owed=owed,
                               extra_cols=extra)
+        elif self.row_norm is not None:
+            # the projection's 32-bit sums are kept up to the norm: biases, the values (which may
+            # be the keys as they stand), the norm over whole rows, rotation and cache write are
+            # one kernel, with one rounding behind it
+            proj = ws.buf("qkv_f32", (n, self.w_qkv.shape[0]), torch.float32)
+            ops.gemm(x, self.w_qkv, proj)
+            qkv = ws.buf("q_rot", (n, H * d), act)
+            ops.rownorm_rope_kvwrite(proj, qkv, step.positions, step.seq_of_token, cos, sin, table,
+                                     layer.k_pages, layer.v_pages, H, KV, d, self.q_norm_w, self.k_norm_w,
+                                     self.dk, self.row_norm[2], q_bias=self.q_bias, k_bias=self.k_bias,
+                                     values_are_keys=self.values_are_keys, write_kv=layer.owns_cache)
         else:
             g0 = (H + (2 * KV if self.own_kv else 0)) * d
             qkv = ws.buf("qkv", (n, self.w_qkv.shape[0]), act)
@@ -376,8 +451,12 @@ class PagedAttention(Mixer):
                 ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
                                  layer.k_pages, layer.v_pages, H, KV, d,
                                  write_kv=layer.owns_cache and self.own_kv)
+        head_gates = None
+        if self.w_head_gate is not None:
+            head_gates = ws.buf("attn_head_gates", (n, self.w_head_gate.shape[0]), torch.float32)
+            ops.gemm(x, self.w_head_gate, head_gates)
         out = ws.buf("attn_out", (n, H * d), act)
-        window = self.window or 0
+        window, chunk = self.window or 0, self.chunk or 0
         bs = layer.k_pages.shape[2]
         work, rows_per_item = self._prefill_work(step, act, bs)
         gate = qkv[:, g0:g0 + H * d] if self.gated else None
@@ -387,7 +466,7 @@ class PagedAttention(Mixer):
             ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
                              work, out, H, KV, d, self.scale, window, self.slopes, rows_per_item,
                              keep_first=self.keep_first, gate=gate_in_kernel, sinks=self.sinks,
-                             score_cap=self.score_cap)
+                             score_cap=self.score_cap, chunk=chunk)
         if step.n_decode:
             splits = self._decode_cuts(step, ops.attention_on_matrix_cores(act, bs))
             workspace = None
@@ -399,7 +478,9 @@ class PagedAttention(Mixer):
                             window, splits, workspace,
                             token_is_seq=step.decode_seq_ids is None and work is None,
                             slopes=self.slopes, keep_first=self.keep_first, gate=gate_in_kernel,
-                            sinks=self.sinks, score_cap=self.score_cap)
+                            sinks=self.sinks, score_cap=self.score_cap, chunk=chunk)
         if gate is not None and gate_in_kernel is None:
             ops.sigmoid_gate(out, gate)
+        if head_gates is not None or self.out_scale != 1.0:
+            ops.head_gate(out, head_gates, H, d, self.out_scale)
         add_product(step, out, self.w_o, residual, owed=owed)

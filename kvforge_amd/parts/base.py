@@ -23,7 +23,8 @@ class WeightSpec:
     """One checkpoint tensor a part expects.
 
     ``init`` drives the random-weights mode: ``"normal"`` draws N(0, std), ``"norm"`` draws
-    1 + N(0, std), ``"zeros"`` is zero.  ``integer`` tensors are tables of int32.  A size of
+    1 + N(0, std), ``"zeros"`` is zero.  ``integer`` tensors are tables of int32 (zeros, or with
+    ``init="choices"`` rows of different numbers below ``int(std)``).  A size of
     ``None`` is one that the checkpoint decides (the part reads it off the tensor it is handed);
     random weights cannot be drawn for such a spec."""
 

@@ -14,19 +14,23 @@ from kvforge_amd.registry import register_block
 
 @register_block("pre_norm")
 class PreNormBlock(Block):
-    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward) -> None:
+    """``ffn`` (and its norm) may be ``None``: a layer of the mixer alone."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None, ffn: FeedForward | None) -> None:
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
 
         self.mixer_takes_residual = self.ffn_takes_residual = False
 
     def parts(self) -> list[Part]:
-        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
 
     def load(self, tensors) -> None:
         super().load(tensors)
         # a part may apply the norm in front of it inside its own first kernel
         self.mixer_takes_residual = self.mixer.absorb_norm(self.mixer_norm)
-        self.ffn_takes_residual = self.ffn.absorb_norm(self.ffn_norm)
+        self.ffn_takes_residual = self.ffn is not None and self.ffn.absorb_norm(self.ffn_norm)
 
     def forward(self, residual, step, layer: LayerState) -> None:
         if self.mixer_takes_residual:
@@ -37,6 +41,8 @@ class PreNormBlock(Block):
             x = step.ws.buf("normed", tuple(residual.shape), step.act_dtype)
             self.mixer_norm.forward(residual, x, add=step.take_owed(residual))
             self.mixer.forward(x, step, layer, residual)
+        if self.ffn is None:
+            return
         if self.ffn_takes_residual:
             if not self.ffn.settles_residual:
                 step.settle()

@@ -161,3 +161,53 @@ class GatedFeedForward(SwiGLU):
         if self.down_bias is not None and not self.defer_down_bias:
             step.settle()
             ops.add_bias(residual, self.down_bias)
+
+
+@register_feed_forward("plain")
+class PlainFeedForward(FeedForward):
+    """``down(act(up x))`` without gate and biases.  ``activation``: ``"relu2"`` (the square of
+    relu), ``"silu"`` or ``"gelu_tanh"``, applied in fp32 to the stored product and rounded once.
+    ``names``: checkpoint names under the prefix, by ``up down``."""
+
+    NAMES = {"up": "up_proj.weight", "down": "down_proj.weight"}
+
+    replayable = True
+
+    def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "relu2",
+                 names: dict[str, str] | None = None) -> None:
+        if activation not in ops.PLAIN_ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {sorted(ops.PLAIN_ACTIVATIONS)}")
+        self.prefix, self.hidden, self.inter = prefix, int(hidden), int(intermediate)
+        self.activation = activation
+        self.names = dict(self.NAMES, **(names or {}))
+        self.w_up: torch.Tensor | None = None
+        self.w_down: torch.Tensor | None = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self._name(self.names["up"]): WeightSpec((self.inter, self.hidden)),
+                self._name(self.names["down"]): WeightSpec((self.hidden, self.inter))}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.w_up = tensors[self._name(self.names["up"])]
+        self.w_down = tensors[self._name(self.names["down"])]
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        return {"elementwise", "gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
+
+    def num_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in map(ops.plain_of, (self.w_up, self.w_down)) if t is not None)
+
+    def held_tensors(self) -> list[torch.Tensor]:
+        return ops.copies_of(self.w_up) + ops.copies_of(self.w_down)
+
+    def seal(self) -> None:
+        self.w_up, self.w_down = ops.streamed(ops.plain_of(self.w_up)), ops.streamed(ops.plain_of(self.w_down))
+
+    def forward(self, x, step, residual) -> None:
+        """``x``: normalised activations."""
+        n = x.shape[0]
+        step.settle()
+        act = step.ws.buf("ffn_act", (n, self.inter), step.act_dtype)
+        ops.gemm(x, self.w_up, act)
+        ops.plain_act(act, act, self.activation)
+        add_product(step, act, self.w_down, residual)

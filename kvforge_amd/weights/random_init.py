@@ -33,6 +33,17 @@ def _sized(name: str, w) -> None:
                          f"model's configuration has to give it")
 
 
+def _choices(w, gen: torch.Generator, device) -> torch.Tensor:
+    """An integer table ``[rows, top]`` whose every row holds ``top`` different numbers below
+    ``int(w.std)``, drawn from ``gen``."""
+    rows, top = w.shape
+    among = int(w.std)
+    if not 0 < top <= among:
+        raise ValueError(f"a table of {top} different choices among {among}")
+    order = torch.rand((rows, among), generator=gen, dtype=torch.float32, device=device).argsort(dim=1)
+    return order[:, :top].to(torch.int32).contiguous()
+
+
 def random_tensors(spec, seed: int, dtype: "str | torch.dtype" = "bfloat16") -> dict[str, torch.Tensor]:
     """Tensors for every name the model expects, drawn in 32-bit in sorted name order from one
     generator and stored as ``dtype`` (the reference draws in 32-bit and casts to the engine's
@@ -42,7 +53,9 @@ def random_tensors(spec, seed: int, dtype: "str | torch.dtype" = "bfloat16") -> 
     out: dict[str, torch.Tensor] = {}
     for name, w in sorted(spec.weight_specs().items()):
         _sized(name, w)
-        if w.integer:
+        if w.integer and w.init == "choices":
+            out[name] = _choices(w, gen, "cpu")
+        elif w.integer:
             out[name] = torch.zeros(w.shape, dtype=torch.int32)
         elif w.init == "zeros":
             out[name] = torch.zeros(w.shape, dtype=store)
@@ -84,7 +97,8 @@ def load_random_weights(spec, seed: int, engine_dtype: torch.dtype, device: "tor
     for name, w in sorted(spec.weight_specs().items()):
         _sized(name, w)
         if w.integer:
-            tensors[name] = torch.zeros(w.shape, dtype=torch.int32, device=device)
+            tensors[name] = (_choices(w, gen, device) if w.init == "choices"
+                             else torch.zeros(w.shape, dtype=torch.int32, device=device))
             continue
         if w.init == "zeros":
             t = torch.zeros(w.shape, dtype=torch.float32, device=device)

@@ -213,6 +213,112 @@ PRESETS["buzinex-1b"] = buzinex_stack(vocab=128256, width=2048, groups=4, heads=
                                       wkv_dim=64, ff=8192)
 
 
+def ludelix(vocab: int, width: int, layers: list, eps: float = 1e-5,
+            max_positions: int | None = None) -> dict[str, Any]:
+    """A Ludelix config.json.  ``layers``: one ``(type, mixer, mlp)`` per layer.  For ``"gla"`` the
+    mixer holds ``heads dim vdim tau`` and ``rank`` (of the gates' two matrices); for
+    ``"attention"`` ``heads kv_heads dim scale`` and optionally ``window``, ``rot_dims``, ``base``
+    and ``scaling`` (``(factor, low, high, original)``); for ``"parallel"`` ``left`` (``heads
+    kv_heads dim vdim scale`` and optionally ``chunk``, ``rot_dims``, ``base``, ``scaling``:
+    ``(factor, original, fast, slow)``), ``right`` (``heads dim vdim decay`` and optionally
+    ``rot_dims``, ``base``), ``left_scale`` and ``right_scale``.  ``mlp``: ``None``, an ``int``
+    (a dense feed-forward of that width) or ``(ff, experts, top, shared_ff)``."""
+    def rot(m: dict, scaling) -> dict | None:
+        if not m.get("rot_dims"):
+            return None
+        out: dict[str, Any] = {"base": float(m.get("base", 10000.0)), "dims": int(m["rot_dims"])}
+        if scaling:
+            out["scaling"] = scaling
+        return out
+
+    out = []
+    for kind, m, mlp in layers:
+        if kind == "gla":
+            mixer: dict[str, Any] = {"dim": m["dim"], "heads": m["heads"], "rank": m["rank"], "tau": float(m["tau"]),
+                                     "vdim": m["vdim"]}
+        elif kind == "attention":
+            sc = m.get("scaling")
+            mixer = {"dim": m["dim"], "heads": m["heads"], "kv_heads": m["kv_heads"], "scale": float(m["scale"]),
+                     "vdim": m["dim"]}
+            if m.get("window"):
+                mixer["mask"] = {"size": m["window"]}
+            r = rot(m, {"factor": float(sc[0]), "low": float(sc[1]), "high": float(sc[2]), "original": int(sc[3])}
+                    if sc else None)
+            if r:
+                mixer["rot"] = r
+        else:
+            lt, rt = m["left"], m["right"]
+            sc = lt.get("scaling")
+            left: dict[str, Any] = {"dim": lt["dim"], "heads": lt["heads"], "kv_heads": lt["kv_heads"],
+                                    "scale": float(lt["scale"]), "vdim": lt["vdim"]}
+            if lt.get("chunk"):
+                left["mask"] = {"size": lt["chunk"]}
+            r = rot(lt, {"factor": float(sc[0]), "original": int(sc[1]), "fast": float(sc[2]), "slow": float(sc[3])}
+                    if sc else None)
+            if r:
+                left["rot"] = r
+            right: dict[str, Any] = {"decay": [float(x) for x in rt["decay"]], "dim": rt["dim"], "heads": rt["heads"],
+                                     "vdim": rt["vdim"]}
+            r = rot(rt, None)
+            if r:
+                right["rot"] = r
+            mixer = {"left": left, "left_scale": float(m.get("left_scale", 1.0)), "right": right,
+                     "right_scale": float(m.get("right_scale", 1.0))}
+        if mlp is None:
+            ff: dict[str, Any] | None = None
+        elif isinstance(mlp, int):
+            ff = {"ff": mlp, "kind": "dense"}
+        else:
+            ff = {"expert": {"ff": mlp[0]}, "kind": "moe", "router": {"experts": mlp[1], "top": mlp[2]}}
+            if mlp[3]:
+                ff["shared"] = {"ff": mlp[3]}
+        out.append({"mixer": mixer, "mlp": ff, "type": kind})
+    cfg: dict[str, Any] = {"architecture": "Ludelix", "layers": out, "norm": {"eps": eps}, "vocab": vocab,
+                           "width": width}
+    if max_positions is not None:
+        cfg["max_positions"] = max_positions
+    return cfg
+
+
+def retention_decays(heads: int) -> list[float]:
+    """One decay per head, ``1 - 2^(-5 - h)``: the usual spread of memory lengths."""
+    return [1.0 - 2.0 ** (-5.0 - h * 6.0 / max(heads - 1, 1)) for h in range(heads)]
+
+
+def ludelix_stack(vocab: int, width: int, groups: int, heads: int, kv_heads: int, dim: int, window: int,
+                  mem_heads: int, mem_dim: int, mem_vdim: int, ff: int, experts: int, top: int, shared_ff: int,
+                  max_positions: int = 131072) -> dict[str, Any]:
+    """``groups`` times (gated linear attention, attention whose values are its keys, chunked
+    attention beside a retention, attention again), the first of each group with a dense
+    feed-forward, the others with experts."""
+    gla = dict(heads=mem_heads, dim=mem_dim, vdim=mem_vdim, tau=16.0, rank=16)
+    att = dict(heads=heads, kv_heads=kv_heads, dim=dim, scale=float(dim) ** -0.5, window=window, rot_dims=dim // 2,
+               base=500000.0, scaling=(8.0, 1.0, 4.0, 8192))
+    par = dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=float(dim) ** -0.5, chunk=window,
+                         rot_dims=dim, base=10000.0, scaling=(8.0, 4096, 32.0, 1.0)),
+               right=dict(heads=mem_heads, dim=mem_dim, vdim=mem_vdim, decay=retention_decays(mem_heads),
+                          rot_dims=mem_dim, base=10000.0), left_scale=1.0, right_scale=1.0)
+    moe = (ff, experts, top, shared_ff)
+    return ludelix(vocab, width, [("gla", gla, top * ff + shared_ff), ("attention", att, moe), ("parallel", par, moe),
+                                  ("attention", att, moe)] * groups, max_positions=max_positions)
+
+
+PRESETS["ludelix-tiny"] = ludelix(
+    vocab=320, width=96,
+    layers=[("gla", dict(heads=2, dim=16, vdim=24, tau=8.0, rank=4), 160),
+            ("attention", dict(heads=4, kv_heads=2, dim=16, scale=0.25, window=24, rot_dims=8,
+                               scaling=(4.0, 1.0, 4.0, 64)), (32, 6, 2, 64)),
+            ("parallel", dict(left=dict(heads=2, kv_heads=1, dim=16, vdim=32, scale=0.25, chunk=20, rot_dims=16,
+                                        scaling=(4.0, 64, 16.0, 1.0)),
+                              right=dict(heads=2, dim=8, vdim=16, decay=[0.9, 0.98], rot_dims=8),
+                              left_scale=1.25, right_scale=0.5), None)],
+    max_positions=1024)
+# layers of the width of llama-1b: what this design's kernels are measured at
+PRESETS["ludelix-1b"] = ludelix_stack(vocab=128256, width=2048, groups=4, heads=32, kv_heads=8, dim=64, window=1024,
+                                      mem_heads=16, mem_dim=64, mem_vdim=128, ff=1024, experts=32, top=4,
+                                      shared_ff=2048)
+
+
 def preset_dict(name: str) -> dict[str, Any]:
     try:
         return dict(PRESETS[name])

@@ -64,7 +64,8 @@ def build_ludelix(cfg: LudelixConfig) -> ModelSpec:
                                q_scale=float(m.dim) ** -0.5, head_weight=True)
         elif layer.type == "attention":
             mixer = attn_cls(f"{p}.mix", w, m.heads, m.kv_heads, m.dim, rotary_of(m.rot), scale=m.scale,
-                             window=m.window, names=ATTENTION_NAMES, row_norm=("q.norm", "k.norm", eps),
+                             window=m.window, value_dim=m.dim, names=ATTENTION_NAMES,
+                             row_norm=("q.norm", "k.norm", eps),
                              bias=("q.b", "k.b"), values_are_keys=True, sink="sink")
         else:
             lt, rt = m.left, m.right

@@ -7,6 +7,7 @@
     python bench.py --phase burst --preset small [--dtype float32]
     python bench.py --phase fogorax [--dtype float32] [--steps 64] [--batch 8]
     python bench.py --phase rudorax [--sizes w1024,w2048] [--steps 64] [--batch 8]
+    python bench.py --phase ludelix [--sizes w1024,w2048] [--steps 64] [--batch 8]
 
 Default run: the layer sizes of Llama 3.2 1B (16 layers, hidden 2048, 32 heads, 8 kv heads, head
 size 64, SwiGLU 8192, vocabulary 128256, llama3 rope scaling, tied embeddings), random weights
@@ -29,6 +30,9 @@ window, the engine's closest existing model.
 ``--phase rudorax`` does the same for the Rudorax design (window attention and matrix-memory
 layers in turn, routed experts), beside a Llama model whose dense feed-forward is as wide as
 what a Rudorax token uses.
+``--phase ludelix`` measures the Ludelix design (gated linear attention, attention whose values
+are its keys, chunked attention beside a retention, experts chosen by a table) beside Rudorax,
+the closest existing model, at equal sizes.
 Peaks are the published MI355X ones: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s
 for fp32.
 """
@@ -571,6 +575,83 @@ def buzinex_points(dtype, batch, prompt_len, steps, warmup, use_graphs=True, onl
     return out
 
 
+# (name, width, q heads, kv heads, head size, memory heads, their key size, their value size,
+#  expert width, experts, chosen, shared width, groups of four layers, vocabulary)
+LUDELIX_SIZES = [("w1024", 1024, 16, 4, 64, 4, 128, 256, 512, 16, 2, 1024, 2, 32000),
+                 ("w2048", 2048, 32, 8, 64, 8, 128, 256, 1024, 32, 4, 2048, 2, 128256),
+                 ("w4096", 4096, 32, 8, 128, 8, 256, 512, 2048, 32, 4, 4096, 1, 128256)]
+LUDELIX_WINDOW, LUDELIX_GATE_RANK = 1024, 16
+
+
+def ludelix_points(dtype, batch, prompt_len, steps, warmup, use_graphs=True, only=None):
+    """Ludelix at a few sizes that resemble a real model's layers (groups of gated linear
+    attention with a dense feed-forward, attention whose values are its keys, chunked attention
+    beside a retention, attention again, the last three with experts chosen by a table), beside
+    the engine's closest existing model, Rudorax, of the same width, heads, window, memory heads,
+    experts and number of layers (window attention and matrix-memory layers in turn, routed
+    experts in all); random weights drawn on the device.  Per size and model: ms per decode step,
+    its share of the HBM roofline, tokens a second of a 2,048-token prefill and its share of the
+    matrix-core peak.  A decode step has to read: the mixers, shared experts and dense
+    feed-forwards once, the experts that the batch's tokens are expected to choose (a share
+    ``1 - (1 - top/experts)^batch`` of them), the keys and values under window and chunk, and
+    every sequence's memories (read and written)."""
+    import torch
+    from kvforge_amd.config.presets import ludelix_stack, rudorax_stack
+
+    elem = 2 if dtype == "bfloat16" else 4
+    out = {}
+    for name, w, H, KV, d, Hm, dk, dv, ff, E, top, shared, groups, vocab in LUDELIX_SIZES:
+        if only and name not in only:
+            continue
+        layers = 4 * groups
+        lud = ludelix_stack(vocab=vocab, width=w, groups=groups, heads=H, kv_heads=KV, dim=d, window=LUDELIX_WINDOW,
+                            mem_heads=Hm, mem_dim=dk, mem_vdim=dv, ff=ff, experts=E, top=top, shared_ff=shared,
+                            max_positions=CONTEXT_CAP)
+        rud = rudorax_stack(vocab=vocab, width=w, pairs=layers // 2, heads=H, kv_heads=KV, dim=d,
+                            window=LUDELIX_WINDOW, lstm_heads=Hm, lstm_dim=dk, lstm_vdim=dv, ff=ff,
+                            experts=E, top=top, identity=0, shared_ff=shared, max_positions=CONTEXT_CAP)
+        routed = 3 * w * ff
+        touched = E * (1.0 - (1.0 - top / E) ** batch)
+        memory = w * Hm * (2 * dk + 3 * dv)                               # q, k, v, gate, output
+        # Ludelix, a group: gla (+ its gates' two matrices) with a dense feed-forward; attention
+        # (q, k, output) twice; chunked attention (q, k, v, output, a gate row per head) beside a retention
+        l_fixed = groups * (memory + LUDELIX_GATE_RANK * (w + Hm * dk) + 2 * w * (top * ff + shared)
+                            + 2 * w * d * (2 * H + KV) + w * d * (2 * H + 2 * KV) + w * H + memory
+                            + 3 * (3 * w * shared + w))
+        l_routed_layers = 3 * groups
+        l_kv = 3 * groups * 2 * KV * d                                     # key and value pages of three layers a group
+        l_state = groups * 2 * Hm * dk * dv * 4 * 2
+        r_fixed = (layers // 2) * (w * d * (2 * H + 2 * KV) + w * (2 * Hm * dk + 3 * Hm * dv + 2 * Hm)) \
+            + layers * (3 * w * shared + w * E)
+        r_kv = (layers // 2) * 2 * KV * d
+        r_state = (layers // 2) * Hm * (dk * dv + dk + 1) * 4 * 2
+        n = PREFILL_TOKENS
+        seen = min(n, LUDELIX_WINDOW)
+        pairs = n * seen - seen * seen / 2.0                               # (query, key) pairs under a window
+        per_model = {
+            "ludelix": (lud, l_fixed, l_routed_layers, l_kv, l_state,
+                        3 * groups * 4.0 * pairs * H * d + 2 * groups * n * Hm * 4.0 * dk * dv),
+            "rudorax": (rud, r_fixed, layers, r_kv, r_state,
+                        (layers // 2) * 4.0 * pairs * H * d + (layers // 2) * n * Hm * 4.0 * dk * dv)}
+        for model, (cfg, fixed, routed_layers, kv, state_bytes, mixing) in per_model.items():
+            need = batch * (prompt_len + steps + warmup + early_tokens(batch, prompt_len) + 32)
+            engine = build_engine(cfg, dtype, batch, max(need, PREFILL_TOKENS + 64), use_graphs=use_graphs)
+            r = decode_run(engine, vocab, batch, prompt_len, steps, warmup)
+            ctx = min(r["mean_ctx"], LUDELIX_WINDOW)
+            s = prefill_run(engine, vocab, PREFILL_TOKENS, repeats=2)
+            read = ((fixed + routed_layers * touched * routed + vocab * w) * elem
+                    + batch * (ctx * kv * elem + state_bytes))
+            flops = 2.0 * n * (fixed + routed_layers * top * routed) + 2.0 * vocab * w + mixing
+            out[f"{name}_{model}"] = {
+                "decode_ms": round(r["ms_per_step"], 4), "decode_tok_s": round(r["tok_s"], 1),
+                "decode_hbm_frac": round(read / (r["seconds"] / steps) / 1e9 / HBM_PEAK_GBS, 4),
+                "prefill_tok_s": round(PREFILL_TOKENS / s, 1), "prefill_ms": round(s * 1e3, 3),
+                "prefill_frac": round(flops / s / MFMA_PEAK[dtype], 4)}
+            del engine
+            torch.cuda.empty_cache()
+    return out
+
+
 def model_numbers(cfg, layers_run):
     h, H, KV, d, I, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
                          cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"])
@@ -599,7 +680,7 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--decode-run-steps", type=int, default=None,
                     help="decode steps the device takes between two looks of the host (engine default: 8)")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products", "fogorax", "rudorax", "buzinex"],
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products", "fogorax", "rudorax", "buzinex", "ludelix"],
                     default="all",
                     help="for profiles: only the decode steps at --batch, or only the prefill; "
                          "mixed: --batch requests with prompts of 128 to 4,096 tokens, chunked "
@@ -610,8 +691,8 @@ def main() -> int:
                          "(launch to launch, so short ones show the host's time); fogorax: the "
                          "Fogorax design at a few layer sizes beside a Llama model of equal sizes; "
                          "rudorax: the Rudorax design likewise (--sizes names some of them); "
-                         "buzinex: the Buzinex design likewise")
-    ap.add_argument("--sizes", default="", help="with --phase rudorax or buzinex: the sizes to run, with commas")
+                         "buzinex: the Buzinex design likewise; ludelix: the Ludelix design beside Rudorax")
+    ap.add_argument("--sizes", default="", help="with --phase rudorax, buzinex or ludelix: the sizes to run, with commas")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -654,6 +735,19 @@ def main() -> int:
                                                     "memory_dim", "ff", "groups", "vocab"), r[1:]))
                                     for r in BUZINEX_SIZES},
                           **buzinex_points(args.dtype, args.batch, args.prompt_len, steps,
+                                           min(args.warmup, 8), not args.no_graphs,
+                                           [x for x in args.sizes.split(",") if x] or None)}))
+        return 0
+    if args.phase == "ludelix":
+        steps = min(args.steps, 64)
+        print(json.dumps({"phase": "ludelix", "dtype": args.dtype, "batch": args.batch,
+                          "prompt_len": args.prompt_len, "steps": steps, "window": LUDELIX_WINDOW,
+                          "prefill_tokens": PREFILL_TOKENS,
+                          "sizes": {r[0]: dict(zip(("width", "heads", "kv_heads", "head_dim", "memory_heads",
+                                                    "memory_dim", "memory_vdim", "expert_ff", "experts", "top",
+                                                    "shared_ff", "groups", "vocab"), r[1:]))
+                                    for r in LUDELIX_SIZES},
+                          **ludelix_points(args.dtype, args.batch, args.prompt_len, steps,
                                            min(args.warmup, 8), not args.no_graphs,
                                            [x for x in args.sizes.split(",") if x] or None)}))
         return 0

@@ -107,6 +107,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
   const int tok = row_ok ? row / G : 0;
   const int head = kvh * G + (row_ok ? row - tok * G : 0);
   const int pos = start + tok;
+  const int first_vis = first_seen(a.window, pos);      // the first key this row sees
   const float slope = a.slopes && row_ok ? a.slopes[head] : 0.f;
   // key ranges: of the workgroup's rows (what is staged) and of this wave's (what it works on)
   int last = item0 + ITEM_ROWS - 1;
@@ -189,7 +190,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
         for (int v = 0; v < 4; ++v) {
           const int j = t0 + 16 * st + 4 * g4 + v;
           bool vis = row_ok && j <= pos && j < ctx;
-          if (a.window != 0) vis = vis && (j >= first_seen(a.window, pos) || j < keep);
+          if (a.window != 0) vis = vis && (j >= first_vis || j < keep);
           sc[v] = vis ? fmaf(slope, static_cast<float>(j - pos), capped(sc[v] * a.scale, a.cap)) : -INFINITY;
           tmax = fmaxf(tmax, sc[v]);
         }

@@ -17,6 +17,8 @@
 //   [num_blocks, KV, d, block_size], so a lane's eight keys of one element are 16 contiguous
 //   bytes.  Probabilities go from the first product's accumulators to the second product's
 //   operand by a rounding to bf16 alone; softmax itself is fp32.
+// (Instead of a window, positions may be cut into chunks counted from position 0 of the sequence,
+// a query then seeing the keys of its own chunk alone: `window` < 0 stands for chunks of -window.)
 // Key j is visible to a query at position p iff j <= p, j < context length and, with a window
 // w > 0, j > p - w or j < keep (the first `keep` keys of a sequence stay visible behind the
 // window).  Scores are scaled after the dot product.
@@ -82,15 +84,21 @@ struct MArgs {
   // a value whose score is not scaled
   const float* sinks;
   float cap;  // 0, or the scaled score s becomes cap * tanh(s / cap) (kernels with BIAS == 2)
+  // window < 0 stands for chunks of c = -window positions, counted from position 0 of the
+  // sequence: a query sees the keys of its own chunk alone.  chunk_magic: floor(2^32 / c), and
+  // 2^32 - 1 for c == 1.
+  unsigned chunk_magic;
 };
 
-// The first key a query at position `pos` sees: with a window w > 0 the key w - 1 before it, with
-// chunks (window < 0, chunks of -window positions counted from position 0) the first key of its
-// own chunk.  It does not fall as `pos` grows, so a range of rows sees from its first row's on.
-__device__ __forceinline__ int first_seen(int window, int pos) {
-  if (window > 0) return pos - window + 1 > 0 ? pos - window + 1 : 0;
-  if (window < 0) return pos - pos % (-window);
-  return 0;
+// The first key of the chunk that position `pos` lies in.  No division: the quotient's estimate
+// mulhi(pos, floor(2^32 / c)) is at most two short, so the remainder is below 3 c and two
+// conditional steps bring it under c.
+__device__ __forceinline__ int chunk_first(const MArgs& a, int pos) {
+  const unsigned c = static_cast<unsigned>(-a.window);
+  unsigned r = static_cast<unsigned>(pos) - __umulhi(static_cast<unsigned>(pos), a.chunk_magic) * c;
+  r = r >= c ? r - c : r;
+  r = r >= c ? r - c : r;
+  return pos - static_cast<int>(r);
 }
 
 // A walk over the blocks of 32 keys that a range of rows sees: blocks counted from `first` up to
@@ -323,7 +331,8 @@ __device__ __forceinline__ uint2 pack4_gated(const f32x4& v, float f, const bf16
 }
 
 // Sets up the rows of `RT` tiles starting at `first_tile`; returns the positions they span.
-template <int DT, int RT>
+// CHUNK: the kernel was built for chunks of positions (a.window < 0) and for nothing else.
+template <int DT, int RT, bool CHUNK = false>
 __device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int q0, int qlen, int start,
                                            int kvh, int first_tile, int j16, int kg, bool seq_ok,
                                            Rows<RT>& rows, bf16x8 (&qf)[RT][(DT + 1) / 2], int& pos_min,
@@ -340,7 +349,8 @@ __device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int 
     rows.head[rt] = kvh * G + (rows.ok[rt] ? row - tok * G : 0);
     {  // the row's position is below the context length, so it is its last visible key
       const int pos = start + tok;
-      const int first = first_seen(a.window, pos);
+      const int first = CHUNK ? chunk_first(a, pos)
+                              : (a.window > 0 && pos - a.window + 1 > 0 ? pos - a.window + 1 : 0);
       rows.first[rt] = rows.ok[rt] ? first : -1;
       rows.span[rt] = rows.ok[rt] ? static_cast<unsigned>(pos - first) : 0u;
       rows.keep[rt] = rows.ok[rt] && a.window > 0 ? min(a.keep, pos + 1) : 0;
@@ -372,6 +382,9 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
     const int* __restrict__ work, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
     bf16_t* __restrict__ out, MArgs a) {
+  // BIAS 3: chunks of positions instead of a window (a.window < 0), scores as with BIAS 0
+  constexpr bool CHUNK = BIAS == 3;
+  constexpr int SCORE = CHUNK ? 0 : BIAS;
   constexpr int DC = (DT + 1) / 2;
   constexpr int N_K = 2 * DC, N_FRAG = N_K + DT;          // fragments of a key block
   constexpr int FPW = (N_FRAG + WAVES - 1) / WAVES;       // fragments a wave stages per block
@@ -403,13 +416,14 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   Rows<RT> rows;
   bf16x8 qf[RT][DC];
   int pos_min, pos_max;
-  setup_rows<DT, RT>(q, a, q0, qlen, start, kvh, wg_tile + wave * RT, j16, kg, seq_ok, rows, qf, pos_min,
+  setup_rows<DT, RT, CHUNK>(q, a, q0, qlen, start, kvh, wg_tile + wave * RT, j16, kg, seq_ok, rows, qf, pos_min,
                      pos_max);
   // key range of this wave, and of the workgroup (tiles wg_tile .. wg_tile + 4*RT - 1)
   int lo_w = 0, hi_w = -1;
   if (pos_max >= 0) {
     hi_w = pos_max < ctx - 1 ? pos_max : ctx - 1;
-    lo_w = first_seen(a.window, pos_min);
+    if (CHUNK) lo_w = chunk_first(a, pos_min);
+    else if (a.window > 0 && pos_min - a.window + 1 > 0) lo_w = pos_min - a.window + 1;
   }
   int lo_g = 0, hi_g = -1;
   if (seq_ok && wg_tile * 16 < qlen * G) {
@@ -417,7 +431,8 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
     if (t_hi > qlen - 1) t_hi = qlen - 1;
     hi_g = start + t_hi < ctx - 1 ? start + t_hi : ctx - 1;
     const int p_lo = start + wg_tile * 16 / G;
-    lo_g = first_seen(a.window, p_lo);
+    if (CHUNK) lo_g = chunk_first(a, p_lo);
+    else if (a.window > 0 && p_lo - a.window + 1 > 0) lo_g = p_lo - a.window + 1;
   }
   const float scale2 = a.scale * LOG2E;
   const int keep_w = a.window > 0 ? a.keep : 0;
@@ -511,8 +526,8 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
             kf[t][c] = as_frag(frag_lds[(buf * N_FRAG + t * DC + c) * KVF_WAVE + lane]);
 #pragma unroll
         for (int t = 0; t < DT; ++t) vf[t] = as_frag(frag_lds[(buf * N_FRAG + N_K + t) * KVF_WAVE + lane]);
-        const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window != 0;
-        block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
+        const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0 || CHUNK;
+        block_update<DT, RT, SCORE>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
       }
     };
     const int kb_first = wk.first;
@@ -595,8 +610,8 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
         for (int c = 0; c < DC; ++c) kf[t][c] = as_frag(keep_first(kr[t][c], kl[t][c]));
 #pragma unroll
       for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(vr[t], vl));
-      const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window != 0;
-      block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
+      const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0 || CHUNK;
+      block_update<DT, RT, SCORE>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc, a.cap);
     }
   }
 
@@ -656,10 +671,15 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
   bf16x8 qf[1][DC];
   int pos_min, pos_max;
   setup_rows<DT, 1>(q, a, q0, qlen, start, kvh, tile, j16, kg, seq_ok, rows, qf, pos_min, pos_max);
+  if (a.window < 0 && rows.ok[0]) {   // chunks of positions: the rows see from their chunk's first key
+    rows.first[0] = chunk_first(a, rows.pos[0]);
+    rows.span[0] = static_cast<unsigned>(rows.pos[0] - rows.first[0]);
+  }
   int lo = 0, hi = -1;
   if (pos_max >= 0) {
     hi = pos_max < ctx - 1 ? pos_max : ctx - 1;
-    lo = first_seen(a.window, pos_min);
+    if (a.window > 0 && pos_min - a.window + 1 > 0) lo = pos_min - a.window + 1;
+    if (a.window < 0) lo = chunk_first(a, pos_min);
   }
   // Blocks of 32 keys go round the waves of all cuts in turn: cut z, wave w take blocks
   // z * NW + w, then every (NW * splits)-th.  Without a window the first block is known before
@@ -862,6 +882,12 @@ bool args_ok(int H, int KV, int d, int bs, int nb, int table_stride, float scale
          static_cast<unsigned long long>(KV) * bs * d / 8 < (1ull << 24);
 }
 unsigned magic_of(int bs) { return static_cast<unsigned>((1ull << 32) / bs) + 1u; }
+// for chunks of c = -window positions: floor(2^32 / c), which for c == 1 is the largest 32-bit number
+unsigned chunk_magic_of(int window) {
+  if (window >= 0) return 0u;
+  const unsigned long long m = (1ull << 32) / static_cast<unsigned long long>(-static_cast<long long>(window));
+  return m > 0xffffffffull ? 0xffffffffu : static_cast<unsigned>(m);
+}
 
 // Row tiles per wave and LDS sharing by head size: what fits the registers and 64 KB of LDS.
 // One tile per wave keeps more workgroups in flight; two halve what a key block costs per row
@@ -879,7 +905,12 @@ void launch_runs_rt(dim3 grid, hipStream_t s, const void* q, const void* k_pages
   constexpr bool SHARE = runs_share(DT);
   constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
   const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
-  if (a.cap > 0.f)   // (never with sinks or slopes: the exported entry refuses the pairs)
+  if (a.window < 0)   // (never with a cap, sinks or slopes: the exported entry refuses the pairs)
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, 3, false>), grid, dim3(256), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), a);
+  else if (a.cap > 0.f)   // (never with sinks or slopes: the exported entry refuses the pairs)
     hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, 2, false>), grid, dim3(256), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
@@ -1015,6 +1046,8 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
   if (num_work <= 0) return 0;
   if (sinks && slopes) return static_cast<int>(hipErrorInvalidValue);   // no kernel has both
   if (!(cap >= 0.f) || (cap > 0.f && (sinks || slopes))) return static_cast<int>(hipErrorInvalidValue);
+  // chunks of positions (window < 0): the kernel for query runs has them with plain scores only
+  if (window < 0 && (sinks || slopes || cap > 0.f)) return static_cast<int>(hipErrorInvalidValue);
   if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
     return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0)
@@ -1026,7 +1059,7 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
   // of one head and finds them in its own L2 after the first workgroup has brought them in.
   const int kv_fastest = num_work <= 65535 ? 1 : 0;
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, keep, kv_fastest, scale, magic_of(bs), slopes,
-                static_cast<const bf16_t*>(gate), gate_stride, sinks, cap};
+                static_cast<const bf16_t*>(gate), gate_stride, sinks, cap, chunk_magic_of(window)};
   const dim3 grid = kv_fastest ? dim3(KV, num_work) : dim3(num_work, KV);
   switch (d / 16) {
 #define GO(DT) \
@@ -1057,7 +1090,7 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
       splits > KVF_WAVE || (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, keep, 0, scale, magic_of(bs), slopes,
-                static_cast<const bf16_t*>(gate), gate_stride, sinks, cap};
+                static_cast<const bf16_t*>(gate), gate_stride, sinks, cap, chunk_magic_of(window)};
   const int G = H / KV, chunks = (G + 15) / 16;
   if (num_seqs > 65535) return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid(KV * chunks, num_seqs, splits);

@@ -1325,7 +1325,8 @@ KVF_EXPORT int kvf_rms_add_norm(int dtype, float* x, const float* y, const float
 //   at once, eps inside the root) and multiplied by weights qw [H dk], kw [KV dk];
 //   the first `rot` elements of every head are rotated in neighbouring pairs by the position's
 //   cos/sin row; q goes to q_out (rounded once), k and v to the token's place in the pages.
-// A workgroup takes a token.
+// A workgroup takes a token, or (blockIdx.y, few tokens) a share of a token's heads after it has
+// summed the whole row's squares for itself.
 template <typename T>
 __global__ __launch_bounds__(256) void rownorm_rope_kvwrite_kernel(
     const float* __restrict__ proj, const float* __restrict__ q_bias, const float* __restrict__ k_bias,
@@ -1351,58 +1352,67 @@ __global__ __launch_bounds__(256) void rownorm_rope_kvwrite_kernel(
       off = p - blk * a.block_size;
     }
   }
+  // the sums of squares over all of q and all of k: a wave a head in turn, its lanes along the
+  // head (no index is divided), the waves' sums joined through LDS
+  const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE, waves = blockDim.x / KVF_WAVE;
   float ssq = 0.f, ssk = 0.f;
-  for (int t = threadIdx.x; t < a.H * dk; t += blockDim.x) {
-    const int hh = t / dk, e = t - hh * dk;
-    const float x = row[hh * a.d + e] + (q_bias ? q_bias[t] : 0.f);
-    ssq = fmaf(x, x, ssq);
-  }
-  for (int t = threadIdx.x; t < a.KV * dk; t += blockDim.x) {
-    const int hh = t / dk, e = t - hh * dk;
-    const float x = row[(a.H + hh) * a.d + e] + (k_bias ? k_bias[t] : 0.f);
-    ssk = fmaf(x, x, ssk);
-  }
-  const float rq = 1.f / sqrtf(block_sum(ssq, scratch[0]) / static_cast<float>(a.H * dk) + eps);
-  const float rk = 1.f / sqrtf(block_sum(ssk, scratch[1]) / static_cast<float>(a.KV * dk) + eps);
-  for (int t = threadIdx.x; t < a.H * d2; t += blockDim.x) {
-    const int hh = t / d2, i = t - hh * d2, e = 2 * i;
+  for (int hh = wave; hh < a.H + a.KV; hh += waves) {
+    const bool is_k = hh >= a.H;
     const float* x = row + hh * a.d;
-    const int wi = hh * dk + e;
-    float y0 = e < dk ? (x[e] + (q_bias ? q_bias[wi] : 0.f)) * rq * qw[wi] : 0.f;
-    float y1 = e + 1 < dk ? (x[e + 1] + (q_bias ? q_bias[wi + 1] : 0.f)) * rq * qw[wi + 1] : 0.f;
-    if (e < a.rot && pos_ok && cs) {
-      const float c = cs[i], sv = sn[i];
-      const float t0 = y0 * c - y1 * sv, t1 = y1 * c + y0 * sv;
-      y0 = t0;
-      y1 = t1;
+    const float* b = is_k ? (k_bias ? k_bias + (hh - a.H) * dk : nullptr) : (q_bias ? q_bias + hh * dk : nullptr);
+    float ss = 0.f;
+    for (int e = lane; e < dk; e += KVF_WAVE) {
+      const float v = x[e] + (b ? b[e] : 0.f);
+      ss = fmaf(v, v, ss);
     }
-    T* dst = q_out + static_cast<size_t>(n) * q_stride + hh * a.d + e;
-    Elem<T>::store(dst, y0);
-    Elem<T>::store(dst + 1, y1);
+    if (is_k) ssk += ss; else ssq += ss;
   }
-  if (page < 0) return;
-  for (int t = threadIdx.x; t < a.KV * d2; t += blockDim.x) {
-    const int hh = t / d2, i = t - hh * d2, e = 2 * i;
-    const float* x = row + (a.H + hh) * a.d;
-    const int wi = hh * dk + e;
-    const float x0 = e < dk ? x[e] + (k_bias ? k_bias[wi] : 0.f) : 0.f;
-    const float x1 = e + 1 < dk ? x[e + 1] + (k_bias ? k_bias[wi + 1] : 0.f) : 0.f;
-    float y0 = e < dk ? x0 * rk * kw[wi] : 0.f;
-    float y1 = e + 1 < dk ? x1 * rk * kw[wi + 1] : 0.f;
-    if (e < a.rot && cs) {
-      const float c = cs[i], sv = sn[i];
-      const float t0 = y0 * c - y1 * sv, t1 = y1 * c + y0 * sv;
-      y0 = t0;
-      y1 = t1;
+  ssq = wave_sum(ssq);
+  ssk = wave_sum(ssk);
+  if (lane == 0) {
+    scratch[0][wave] = ssq;
+    scratch[1][wave] = ssk;
+  }
+  __syncthreads();
+  float tq = 0.f, tk = 0.f;
+  for (int w = 0; w < waves; ++w) {
+    tq += scratch[0][w];
+    tk += scratch[1][w];
+  }
+  const float rq = 1.f / sqrtf(tq / static_cast<float>(a.H * dk) + eps);
+  const float rk = 1.f / sqrtf(tk / static_cast<float>(a.KV * dk) + eps);
+  // a wave a head in turn (blockIdx.y names a share of the heads); a lane holds the pairs lane and lane + 64
+  for (int hh = blockIdx.y * waves + wave; hh < a.H + a.KV; hh += gridDim.y * waves) {
+    const bool is_k = hh >= a.H;
+    if (is_k && page < 0) continue;
+    const int kh = hh - a.H;
+    const float* x = row + hh * a.d;
+    const float* b = is_k ? (k_bias ? k_bias + kh * dk : nullptr) : (q_bias ? q_bias + hh * dk : nullptr);
+    const float* w = is_k ? kw + kh * dk : qw + hh * dk;
+    const float r = is_k ? rk : rq;
+    T* dst = is_k ? k_pages + ((static_cast<size_t>(page) * a.KV + kh) * a.block_size + off) * a.d
+                  : q_out + static_cast<size_t>(n) * q_stride + hh * a.d;
+    const float* vx = row + (a.H + a.KV + (is_k ? kh : 0)) * a.d;
+    T* vdst = is_k ? v_pages + (static_cast<size_t>(page) * a.KV + kh) * a.d * a.block_size + off : nullptr;
+    for (int i = lane; i < d2; i += KVF_WAVE) {
+      const int e = 2 * i;
+      const float x0 = e < dk ? x[e] + (b ? b[e] : 0.f) : 0.f;
+      const float x1 = e + 1 < dk ? x[e + 1] + (b ? b[e + 1] : 0.f) : 0.f;
+      float y0 = e < dk ? x0 * r * w[e] : 0.f;
+      float y1 = e + 1 < dk ? x1 * r * w[e + 1] : 0.f;
+      if (e < a.rot && pos_ok && cs) {
+        const float c = cs[i], sv = sn[i];
+        const float t0 = y0 * c - y1 * sv, t1 = y1 * c + y0 * sv;
+        y0 = t0;
+        y1 = t1;
+      }
+      Elem<T>::store(dst + e, y0);
+      Elem<T>::store(dst + e + 1, y1);
+      if (is_k) {
+        Elem<T>::store(vdst + static_cast<size_t>(e) * a.block_size, v_from_k ? x0 : vx[e]);
+        Elem<T>::store(vdst + static_cast<size_t>(e + 1) * a.block_size, v_from_k ? x1 : vx[e + 1]);
+      }
     }
-    T* dst = k_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.block_size + off) * a.d + e;
-    Elem<T>::store(dst, y0);
-    Elem<T>::store(dst + 1, y1);
-    const float* vx = row + (a.H + a.KV + hh) * a.d;
-    const float v0 = v_from_k ? x0 : vx[e], v1 = v_from_k ? x1 : vx[e + 1];
-    T* vdst = v_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.d + e) * a.block_size + off;
-    Elem<T>::store(vdst, v0);
-    Elem<T>::store(vdst + a.block_size, v1);
   }
 }
 #define ROWNORM_ARGS_DECL                                                                                    \
@@ -1417,12 +1427,16 @@ KVF_EXPORT int kvf_rownorm_rope_kvwrite(ROWNORM_ARGS_DECL) {
   if (d % 2 || dk > d || dk <= 0 || rot > dk || rot % 2 || !qw || !kw || !q_out)
     return static_cast<int>(hipErrorInvalidValue);
   const RopeArgs a{ROPE_ARGS_PACK};
+  // few tokens: several workgroups share a token's pairs, so that the chip has work
+  int shares = n >= 1024 ? 1 : (H + KV + 3) / 4;
+  if (shares > 64) shares = 64;
+  const dim3 grid(n, shares);
   if (dtype == 0)
-    hipLaunchKernelGGL(rownorm_rope_kvwrite_kernel<float>, dim3(n), dim3(256), 0, s, proj, q_bias, k_bias, qw, kw,
+    hipLaunchKernelGGL(rownorm_rope_kvwrite_kernel<float>, grid, dim3(256), 0, s, proj, q_bias, k_bias, qw, kw,
                        positions, seq_of_token, cos_t, sin_t, block_table, static_cast<float*>(q_out), q_stride,
                        static_cast<float*>(k_pages), static_cast<float*>(v_pages), dk, eps, v_from_k, a);
   else if (dtype == 1)
-    hipLaunchKernelGGL(rownorm_rope_kvwrite_kernel<bf16_t>, dim3(n), dim3(256), 0, s, proj, q_bias, k_bias, qw, kw,
+    hipLaunchKernelGGL(rownorm_rope_kvwrite_kernel<bf16_t>, grid, dim3(256), 0, s, proj, q_bias, k_bias, qw, kw,
                        positions, seq_of_token, cos_t, sin_t, block_table, static_cast<bf16_t*>(q_out), q_stride,
                        static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages), dk, eps, v_from_k, a);
   else
@@ -1476,8 +1490,31 @@ __global__ void plain_act_kernel(const T* __restrict__ x, T* __restrict__ out, s
   const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i < total) Elem<T>::store(out + i, plain_act_f(act, Elem<T>::load(x + i)));
 }
+// eight neighbouring elements a thread (16 bytes of bf16 in and out)
+template <typename T>
+__global__ void plain_act8_kernel(const T* __restrict__ x, T* __restrict__ out, size_t groups, int act) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= groups) return;
+  float v[8];
+  load8(x + 8 * i, v);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = plain_act_f(act, v[e]);
+  store8(out + 8 * i, v);
+}
 KVF_EXPORT int kvf_plain_act(int dtype, const void* x, void* out, long total, int act, hipStream_t s) {
   if (total <= 0) return 0;
+  if (total % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 32 == 0 && reinterpret_cast<uintptr_t>(out) % 32 == 0 &&
+      dtype >= 0 && dtype <= 1) {
+    const size_t groups = static_cast<size_t>(total / 8);
+    const dim3 grid8(static_cast<unsigned>((groups + 255) / 256));
+    if (dtype == 0)
+      hipLaunchKernelGGL(plain_act8_kernel<float>, grid8, dim3(256), 0, s, static_cast<const float*>(x),
+                         static_cast<float*>(out), groups, act);
+    else
+      hipLaunchKernelGGL(plain_act8_kernel<bf16_t>, grid8, dim3(256), 0, s, static_cast<const bf16_t*>(x),
+                         static_cast<bf16_t*>(out), groups, act);
+    return kvf_last_error();
+  }
   const dim3 grid(static_cast<unsigned>((total + 255) / 256));
   if (dtype == 0)
     hipLaunchKernelGGL(plain_act_kernel<float>, grid, dim3(256), 0, s, static_cast<const float*>(x),

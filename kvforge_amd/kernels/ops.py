@@ -1198,6 +1198,9 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         rows_per_item = prefill_rows_per_item(q.dtype, d, bs)
     _no_sinks_with_slopes(sinks, slopes, attention_on_matrix_cores(q.dtype, bs))
     if attention_on_matrix_cores(q.dtype, bs):
+        if window < 0 and (sinks is not None or slopes is not None or cap > 0.0):
+            raise KernelError("attn_prefill: the matrix-core kernel has chunks of positions with plain scores "
+                              "only (no sinks, slopes or score cap beside them)")
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
                 [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p])
         _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),

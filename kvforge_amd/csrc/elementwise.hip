@@ -1459,10 +1459,38 @@ __global__ void head_gate_kernel(T* __restrict__ y, const float* __restrict__ g,
   const float gate = g ? 1.f / (1.f + expf(-g[m * g_stride + c / d])) : 1.f;
   Elem<T>::store(yp, Elem<T>::load(yp) * (gate * scale));
 }
+// eight neighbouring elements of one head a thread (d a multiple of 8, rows that start on 16 / 32 bytes)
+template <typename T>
+__global__ void head_gate8_kernel(T* __restrict__ y, const float* __restrict__ g, int H, int d, int y_stride,
+                                  int g_stride, float scale, int rows) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (c >= H * d) return;
+  const int head = c / d;
+  for (int m = blockIdx.y; m < rows; m += gridDim.y) {
+    const float gate = g ? 1.f / (1.f + expf(-g[static_cast<size_t>(m) * g_stride + head])) : 1.f;
+    T* yp = y + static_cast<size_t>(m) * y_stride + c;
+    float v[8];
+    load8(yp, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] *= gate * scale;
+    store8(yp, v);
+  }
+}
 KVF_EXPORT int kvf_head_gate(int dtype, void* y, const float* g, int m, int H, int d, int y_stride, int g_stride,
                              float scale, hipStream_t s) {
   const size_t total = static_cast<size_t>(m) * H * d;
   if (total == 0) return 0;
+  if (d % 8 == 0 && y_stride % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 32 == 0 && (dtype == 0 || dtype == 1)) {
+    const int threads = H * d / 8 >= 256 ? 256 : 64;
+    const dim3 grid8((H * d / 8 + threads - 1) / threads, m < 65535 ? m : 65535);
+    if (dtype == 0)
+      hipLaunchKernelGGL(head_gate8_kernel<float>, grid8, dim3(threads), 0, s, static_cast<float*>(y), g, H, d,
+                         y_stride, g_stride, scale, m);
+    else
+      hipLaunchKernelGGL(head_gate8_kernel<bf16_t>, grid8, dim3(threads), 0, s, static_cast<bf16_t*>(y), g, H, d,
+                         y_stride, g_stride, scale, m);
+    return kvf_last_error();
+  }
   const dim3 grid(static_cast<unsigned>((total + 255) / 256));
   if (dtype == 0)
     hipLaunchKernelGGL(head_gate_kernel<float>, grid, dim3(256), 0, s, static_cast<float*>(y), g, H, d, y_stride,
@@ -1543,10 +1571,37 @@ __global__ void gated_act_rowgate_kernel(const T* __restrict__ gu, const float* 
   const float z = rg[m * rg_stride];
   Elem<T>::store(out + idx, act_f(act, g) * u * (1.f / (1.f + expf(-z))));
 }
+// bf16: a thread takes four neighbouring (gate, up) pairs (16 bytes in, 8 bytes out); the grid's x
+// runs along a row, its y over the rows
+__global__ void gated_act_rowgate4_kernel(const bf16_t* __restrict__ gu, const float* __restrict__ rg, int rg_stride,
+                                          bf16_t* __restrict__ out, int inter, int rows, int act) {
+  const int i0 = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i0 >= inter) return;
+  for (int m = blockIdx.y; m < rows; m += gridDim.y) {
+    const float gate = 1.f / (1.f + expf(-rg[static_cast<size_t>(m) * rg_stride]));
+    float v[8];
+    load8(gu + (static_cast<size_t>(m) * inter + i0) * 2, v);
+    uint32_t hh[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) hh[i] = f32_to_bf16(act_f(act, v[2 * i]) * v[2 * i + 1] * gate);
+    uint2 packed;
+    packed.x = hh[0] | (hh[1] << 16);
+    packed.y = hh[2] | (hh[3] << 16);
+    *reinterpret_cast<uint2*>(out + static_cast<size_t>(m) * inter + i0) = packed;
+  }
+}
 KVF_EXPORT int kvf_gated_act_rowgate(int dtype, const void* gu, const float* rg, int rg_stride, void* out, int m,
                                      int inter, int act, hipStream_t s) {
   const size_t total = static_cast<size_t>(m) * inter;
   if (total == 0) return 0;
+  if (dtype == 1 && inter % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 8 == 0) {
+    const int threads = inter / 4 >= 256 ? 256 : 64;
+    const dim3 grid4((inter / 4 + threads - 1) / threads, m < 65535 ? m : 65535);
+    hipLaunchKernelGGL(gated_act_rowgate4_kernel, grid4, dim3(threads), 0, s, static_cast<const bf16_t*>(gu), rg,
+                       rg_stride, static_cast<bf16_t*>(out), inter, m, act);
+    return kvf_last_error();
+  }
   const dim3 grid(static_cast<unsigned>((total + 255) / 256));
   if (dtype == 0)
     hipLaunchKernelGGL(gated_act_rowgate_kernel<float>, grid, dim3(256), 0, s, static_cast<const float*>(gu), rg,

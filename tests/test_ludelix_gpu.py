@@ -147,7 +147,7 @@ def test_a_window_and_chunks_exclude_each_other():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,d", [(1, 16), (5, 24), (8, 64)])
+@pytest.mark.parametrize("H,d", [(1, 16), (5, 24), (8, 64), (3, 10), (2, 36)])
 def test_one_gate_per_head_and_a_constant(dtype, H, d):
     y = rand(9, H * d + 8, seed=H).to(dtype)
     g = rand(9, 16, seed=d, scale=2.0)
@@ -166,12 +166,17 @@ def test_squared_relu_and_a_gate_per_row(dtype):
     dev = x.clone().to(DEV)
     ops().plain_act(dev, dev, "relu2")
     torch.testing.assert_close(dev.float().cpu(), torch.relu(x.float()) ** 2, **tol(dtype))
-    gu, rg = rand(7, 60, seed=2).to(dtype), rand(7, 16, seed=3, scale=2.0)
-    out = torch.zeros(7, 30, dtype=dtype, device=DEV)
-    ops().gated_act_rowgate(gu.to(DEV), rg.to(DEV), out, "silu")
-    g, u = gu.float()[:, 0::2], gu.float()[:, 1::2]
-    want = torch.nn.functional.silu(g) * u * torch.sigmoid(rg[:, :1])
-    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    for inter in (30, 32, 1024):              # one pair a thread, and four
+        gu, rg = rand(7, 2 * inter, seed=2).to(dtype), rand(7, 16, seed=3, scale=2.0)
+        out = torch.zeros(7, inter, dtype=dtype, device=DEV)
+        ops().gated_act_rowgate(gu.to(DEV), rg.to(DEV), out, "silu")
+        g, u = gu.float()[:, 0::2], gu.float()[:, 1::2]
+        want = torch.nn.functional.silu(g) * u * torch.sigmoid(rg[:, :1])
+        torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    wide = rand(5, 4096, seed=4, scale=2.0).to(dtype).to(DEV)      # eight elements a thread
+    into = torch.zeros_like(wide)
+    ops().plain_act(wide, into, "relu2")
+    torch.testing.assert_close(into.float().cpu(), torch.relu(wide.float().cpu()) ** 2, **tol(dtype))
 
 
 def test_a_table_chooses_the_experts():
